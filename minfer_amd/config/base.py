@@ -104,11 +104,14 @@ def read_config_json(folder_or_file: str) -> Dict[str, Any]:
 
 
 def architecture_name(raw: Dict[str, Any]) -> str:
-    """The model class a config.json asks for: architectures[0]."""
+    """The model class a config.json asks for: architectures[0], or the single name under
+    `architecture` where a design's files say it that way."""
     archs = raw.get("architectures")
+    if archs is None:
+        archs = raw.get("architecture")
     if isinstance(archs, str):
         return archs
     if isinstance(archs, (list, tuple)) and archs and isinstance(archs[0], str):
         return archs[0]
-    raise ConfigError("config.json: 'architectures' must be a non-empty list of names, "
-                      f"found {archs!r}")
+    raise ConfigError("config.json: 'architectures' must be a non-empty list of names (or 'architecture' "
+                      f"a name), found {archs!r}")

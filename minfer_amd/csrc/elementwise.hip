@@ -104,6 +104,86 @@ MF_API int mf_rmsnorm(const float* x, const int* row_idx, const float* w, void* 
   return mf_launch_status();
 }
 
+// ---------------------------------------------------------------- RMS norm in groups
+// The row is cut into `groups` equal consecutive parts; each part is divided by its own
+// sqrt(mean(part^2) + eps) and the whole is multiplied by w.  Three uses of one kernel:
+// write the normed row (run type), add it into a 32-bit row (a residual stream that takes a
+// branch's normed output: h += N(y)), and, with the sum, leave the new row rounded to bfloat16
+// as well for the product that reads the stream next.  x and out may be the same rows (a part is
+// summed before any of it is written).
+template <typename OT, bool ADD>
+__global__ __launch_bounds__(256) void group_rmsnorm_kernel(const float* x,
+                                                            const int* __restrict__ row_idx,
+                                                            const float* __restrict__ w, OT* out,
+                                                            bf16* __restrict__ cast_out, int d, int groups,
+                                                            float eps) {
+  __shared__ float scratch[4];
+  const int row = blockIdx.x;
+  const float* xr = x + (size_t)(row_idx ? row_idx[row] : row) * d;
+  OT* o = out + (size_t)row * d;
+  bf16* co = cast_out ? cast_out + (size_t)row * d : nullptr;
+  const int part = d / groups;
+  for (int g = 0; g < groups; ++g) {
+    const int lo = g * part;
+    float ss = 0.f;
+    for (int i = threadIdx.x; i < part; i += 256) {
+      const float v = xr[lo + i];
+      ss = fmaf(v, v, ss);
+    }
+    ss = block_sum<256>(ss, scratch);
+    const float scale = 1.0f / sqrtf(ss / (float)part + eps);
+    for (int i = threadIdx.x; i < part; i += 256) {
+      float y = xr[lo + i] * scale * (w ? w[lo + i] : 1.0f);
+      if (ADD) y += to_f32(o[lo + i]);
+      o[lo + i] = from_f32<OT>(y);
+      if (co) co[lo + i] = (bf16)y;
+    }
+    __syncthreads();
+  }
+}
+
+MF_API int mf_group_rmsnorm(const float* x, const int* row_idx, const float* w, void* out, int out_is_bf16,
+                            int add, void* cast_out, int rows, int d, int groups, float eps,
+                            hipStream_t stream) {
+  if (rows <= 0) return 0;
+  if (groups < 1 || d % groups != 0 || (add && out_is_bf16)) return (int)hipErrorInvalidValue;
+  if (add)
+    group_rmsnorm_kernel<float, true><<<rows, 256, 0, stream>>>(x, row_idx, w, (float*)out, (bf16*)cast_out, d,
+                                                                 groups, eps);
+  else if (out_is_bf16)
+    group_rmsnorm_kernel<bf16, false><<<rows, 256, 0, stream>>>(x, row_idx, w, (bf16*)out, (bf16*)cast_out, d,
+                                                                 groups, eps);
+  else
+    group_rmsnorm_kernel<float, false><<<rows, 256, 0, stream>>>(x, row_idx, w, (float*)out, (bf16*)cast_out, d,
+                                                                  groups, eps);
+  return mf_launch_status();
+}
+
+// ---------------------------------------------------------------- xIELU
+// z > 0: a_pos z^2 + z/2;  z <= 0: a_neg (e^z - 1 - z) + z/2, where a_pos = softplus(p) and
+// a_neg = 1/2 + softplus(q) come from the layer's two learned numbers (the host works them out).
+__device__ __forceinline__ float xielu_of(float z, float a_pos, float a_neg) {
+  return z > 0.f ? fmaf(a_pos * z, z, 0.5f * z) : fmaf(a_neg, expm1f(z) - z, 0.5f * z);
+}
+
+template <typename OT>
+__global__ __launch_bounds__(256) void xielu_kernel(const float* __restrict__ x, OT* __restrict__ out, size_t n,
+                                                    float a_pos, float a_neg) {
+  const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (i < n) out[i] = from_f32<OT>(xielu_of(x[i], a_pos, a_neg));
+}
+
+MF_API int mf_xielu(const float* x, void* out, int out_is_bf16, size_t n, float a_pos, float a_neg,
+                    hipStream_t stream) {
+  if (n == 0) return 0;
+  const unsigned blocks = (unsigned)((n + 255) / 256);
+  if (out_is_bf16)
+    xielu_kernel<bf16><<<blocks, 256, 0, stream>>>(x, (bf16*)out, n, a_pos, a_neg);
+  else
+    xielu_kernel<float><<<blocks, 256, 0, stream>>>(x, (float*)out, n, a_pos, a_neg);
+  return mf_launch_status();
+}
+
 // out[r][:] = x[idx[r]][:]  (generic row selection, src/graph/cpu_backend.rs:255-268)
 __global__ __launch_bounds__(256) void gather_rows_kernel(const float* __restrict__ x,
                                                           const int* __restrict__ idx,
@@ -194,6 +274,27 @@ MF_API int mf_rope_table(float* cs, float* sn, int n_pos, int half, double theta
   const int n = n_pos * half;
   if (n <= 0) return 0;
   rope_table_kernel<<<(n + 255) / 256, 256, 0, stream>>>(cs, sn, n_pos, half, theta, freq_scale);
+  return mf_launch_status();
+}
+
+// cos and sin of position * freq[i], times `magnitude`, for frequencies the host has worked out
+// in double (any ladder: plain, blended towards longer periods, ...): [n_pos][half].
+__global__ __launch_bounds__(256) void rope_table_freqs_kernel(float* __restrict__ cs, float* __restrict__ sn,
+                                                               const double* __restrict__ freqs, int n_pos,
+                                                               int half, double magnitude) {
+  const int idx = blockIdx.x * 256 + threadIdx.x;
+  if (idx >= n_pos * half) return;
+  const int pos = idx / half, i = idx % half;
+  const double ang = (double)pos * freqs[i];
+  cs[idx] = (float)(cos(ang) * magnitude);
+  sn[idx] = (float)(sin(ang) * magnitude);
+}
+
+MF_API int mf_rope_table_freqs(float* cs, float* sn, const double* freqs, int n_pos, int half,
+                               double magnitude, hipStream_t stream) {
+  const int n = n_pos * half;
+  if (n <= 0) return 0;
+  rope_table_freqs_kernel<<<(n + 255) / 256, 256, 0, stream>>>(cs, sn, freqs, n_pos, half, magnitude);
   return mf_launch_status();
 }
 
@@ -334,6 +435,33 @@ MF_API int mf_rope_inplace(float* x, const float* cs, const float* sn, const int
   if (n_tok <= 0 || n_rot <= 0) return 0;
   if (hd % 2 != 0 || n_rot > n_heads_total || !cs || !sn) return (int)hipErrorInvalidValue;
   rope_inplace_kernel<<<n_tok, 256, 0, stream>>>(x, cs, sn, positions, n_rot, n_heads_total, hd);
+  return mf_launch_status();
+}
+
+// The rotation in neighbouring pairs (2i, 2i+1), in place: the first 2 `half` values of each of the
+// first n_rot heads are rotated, whatever lies behind them in the head passes unchanged.
+__global__ __launch_bounds__(256) void rope_pairs_inplace_kernel(float* __restrict__ x, const float* __restrict__ cs,
+                                                                 const float* __restrict__ sn,
+                                                                 const int* __restrict__ positions, int n_rot,
+                                                                 int n_heads_total, int hd, int half) {
+  const int t = blockIdx.x;
+  const int pos = positions[t];
+  float* row = x + (size_t)t * n_heads_total * hd;
+  for (int it = threadIdx.x; it < n_rot * half; it += 256) {
+    const int head = it / half, i = it % half;
+    const float c = cs[(size_t)pos * half + i], s = sn[(size_t)pos * half + i];
+    float* p = row + (size_t)head * hd + 2 * i;
+    const float x0 = p[0], x1 = p[1];
+    p[0] = x0 * c - x1 * s;
+    p[1] = x1 * c + x0 * s;
+  }
+}
+
+MF_API int mf_rope_pairs_inplace(float* x, const float* cs, const float* sn, const int* positions, int n_tok,
+                                 int n_rot, int n_heads_total, int hd, int half, hipStream_t stream) {
+  if (n_tok <= 0 || n_rot <= 0 || half <= 0) return 0;
+  if (2 * half > hd || n_rot > n_heads_total || !cs || !sn) return (int)hipErrorInvalidValue;
+  rope_pairs_inplace_kernel<<<n_tok, 256, 0, stream>>>(x, cs, sn, positions, n_rot, n_heads_total, hd, half);
   return mf_launch_status();
 }
 

@@ -30,6 +30,8 @@ LIBRARIES: Dict[str, str] = {
     "attn_tokens_f32": "attn_tokens_f32.hip",
     "attn_decode_bf16": "attn_decode_bf16.hip",
     "attn_prefill_bf16": "attn_prefill_bf16.hip",
+    "attn_latent": "attn_latent.hip",
+    "recurrence": "recurrence.hip",
     "sampling": "sampling.hip",
     "probe": "probe.hip",
 }

@@ -39,6 +39,22 @@ _PROTOTYPES = {
                             c_int, c_int, _P],
         "mf_rope_inplace": [_P, _P, _P, _P, c_int, c_int, c_int, c_int, _P],
         "mf_fill_normal": [_P, c_int, c_size_t, c_uint64, c_float, c_int, _P],
+        "mf_group_rmsnorm": [_P, _P, _P, _P, c_int, c_int, _P, c_int, c_int, c_int, c_float, _P],
+        "mf_xielu": [_P, _P, c_int, c_size_t, c_float, c_float, _P],
+        "mf_rope_table_freqs": [_P, _P, _P, c_int, c_int, c_double, _P],
+        "mf_rope_pairs_inplace": [_P, _P, _P, _P, c_int, c_int, c_int, c_int, c_int, _P],
+    },
+    "recurrence": {
+        "mf_mingru_scan": [_P, _P, _P, _P, _P, c_int, c_int, c_int, _P],
+        "mf_mingru_scan_chunked": [_P, _P, c_int, _P, _P, _P, _P, _P, c_int, c_int, c_int, _P],
+        "mf_scan_chunk": [],
+    },
+    "attn_latent": {
+        "mf_latent_prep": [_P, c_int, c_int, c_int, _P, c_float, _P, _P, c_int, _P, _P, _P, c_int, _P, _P, _P, _P,
+                           c_int, c_int, c_int, c_int, c_int, c_int, c_int, _P],
+        "mf_headwise_linear": [_P, c_int, _P, _P, c_int, _P, c_int, c_int, c_int, c_int, c_int, _P],
+        "mf_latent_attn": [_P, _P, _P, c_int, _P, _P, _P, _P, c_int, c_int, c_int, c_int, c_int, c_float, c_int,
+                           c_int, c_int, _P],
     },
     "probe": {
         "mf_probe_read": [_P, c_size_t, _P, c_int, _P],
@@ -403,6 +419,223 @@ def rope_kvwrite(qkv: torch.Tensor, cos: Optional[torch.Tensor], sin: Optional[t
         page_table.shape[1], _ptr(q_out), _ptr(kcache if write_kv else None),
         _ptr(vcache if write_kv else None), _is_bf16(q_out), n_tok, n_heads, n_kv_heads, head_dim,
         1 if write_kv else 0, _stream()), "rope_kvwrite")
+
+
+# ------------------------------------------------------------------ norm in groups, xIELU, frequency tables
+def group_rmsnorm(x: torch.Tensor, weight: Optional[torch.Tensor], eps: float, groups: int, out: torch.Tensor,
+                  row_idx: Optional[torch.Tensor] = None, add: bool = False,
+                  cast_out: Optional[torch.Tensor] = None) -> None:
+    """The RMS norm taken over `groups` equal consecutive parts of each row, times `weight`.
+    `out` gets the normed rows (run type); with `add` they are added into the float32 `out` instead
+    (a residual stream taking a branch's normed result), and `cast_out` (bfloat16) then also gets the
+    new rows rounded.  `x` and `out` may be the same tensor."""
+    _need(x, "group_rmsnorm.x", torch.float32)
+    d = x.shape[-1]
+    rows = out.shape[0]
+    _need(out, "group_rmsnorm.out", torch.float32 if add else _FLOATS, (rows, d))
+    if groups < 1 or d % groups:
+        raise KernelError(f"group_rmsnorm: {d} values do not split into {groups} equal parts")
+    if weight is not None:
+        _need(weight, "group_rmsnorm.weight", torch.float32, (d,))
+    if row_idx is not None:
+        _need(row_idx, "group_rmsnorm.row_idx", torch.int32, (rows,))
+    elif x.shape[0] != rows:
+        raise KernelError(f"group_rmsnorm: x has {x.shape[0]} rows, out has {rows}")
+    if cast_out is not None:
+        _need(cast_out, "group_rmsnorm.cast_out", torch.bfloat16, (rows, d))
+    _check(_fn("elementwise", "mf_group_rmsnorm")(_ptr(x), _ptr(row_idx), _ptr(weight), _ptr(out), _is_bf16(out),
+                                                   1 if add else 0, _ptr(cast_out), rows, d, int(groups), float(eps),
+                                                   _stream()), "group_rmsnorm")
+
+
+def xielu(x: torch.Tensor, out: torch.Tensor, a_pos: float, a_neg: float) -> None:
+    """out = a_pos x^2 + x/2 where x > 0, a_neg (e^x - 1 - x) + x/2 elsewhere; x float32, out run type."""
+    _need(x, "xielu.x", torch.float32)
+    _need(out, "xielu.out", _FLOATS, tuple(x.shape))
+    _check(_fn("elementwise", "mf_xielu")(_ptr(x), _ptr(out), _is_bf16(out), x.numel(), float(a_pos), float(a_neg),
+                                           _stream()), "xielu")
+
+
+def rope_table_freqs(n_pos: int, freqs, magnitude: float, device):
+    """(cos, sin) float32 `[n_pos][len(freqs)]` of position * freqs[i], both times `magnitude`;
+    the frequencies are given in double and the angles are formed in double on the device."""
+    f = torch.tensor([float(v) for v in freqs], dtype=torch.float64).to(device)
+    half = f.numel()
+    cs = torch.empty((n_pos, half), dtype=torch.float32, device=device)
+    sn = torch.empty((n_pos, half), dtype=torch.float32, device=device)
+    _need(cs, "rope_table_freqs.out")
+    _check(_fn("elementwise", "mf_rope_table_freqs")(_ptr(cs), _ptr(sn), _ptr(f), n_pos, half, float(magnitude),
+                                                      _stream()), "rope_table_freqs")
+    return cs, sn
+
+
+def rope_pairs_inplace(qkv: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor, positions: torch.Tensor,
+                       n_rot_heads: int, n_heads_total: int, head_dim: int) -> None:
+    """The rotation in neighbouring pairs alone: values (2i, 2i+1), i below the tables' width, of the
+    first `n_rot_heads` heads of every token's `[n_heads_total][head_dim]` row of 32-bit values are
+    rotated in place; the rest of a head passes unchanged."""
+    n_tok = positions.numel()
+    _need(qkv, "rope_pairs_inplace.qkv", torch.float32, (n_tok, n_heads_total * head_dim))
+    _need(cos, "rope_pairs_inplace.cos", torch.float32)
+    _need(sin, "rope_pairs_inplace.sin", torch.float32, tuple(cos.shape))
+    if 2 * cos.shape[1] > head_dim or n_rot_heads > n_heads_total:
+        raise KernelError(f"rope_pairs_inplace: table {tuple(cos.shape)}, head_dim {head_dim}, "
+                          f"{n_rot_heads} of {n_heads_total} heads")
+    _need(positions, "rope_pairs_inplace.positions", torch.int32, (n_tok,))
+    _check(_fn("elementwise", "mf_rope_pairs_inplace")(_ptr(qkv), _ptr(cos), _ptr(sin), _ptr(positions), n_tok,
+                                                        n_rot_heads, n_heads_total, head_dim, cos.shape[1],
+                                                        _stream()), "rope_pairs_inplace")
+
+
+# ------------------------------------------------------------------ recurrences
+SCAN_CHUNK = 64          # tokens of a chunk of the chunked scan (MF_SCAN_CHUNK in csrc/recurrence.hip)
+
+
+def scan_chunks(host_new):
+    """The chunk table of the chunked scan for a step whose sequences bring `host_new` tokens:
+    int32 `[5][n_chunks]` (first token, tokens, sequence, first chunk of the sequence, last or not)."""
+    t0s, ns, seqs, firsts, lasts = [], [], [], [], []
+    t = 0
+    for b, n in enumerate(host_new):
+        first = len(t0s)
+        for c0 in range(0, n, SCAN_CHUNK):
+            t0s.append(t + c0)
+            ns.append(min(SCAN_CHUNK, n - c0))
+            seqs.append(b)
+            firsts.append(first)
+            lasts.append(1 if c0 + SCAN_CHUNK >= n else 0)
+        t += n
+    return torch.tensor([t0s, ns, seqs, firsts, lasts], dtype=torch.int32)
+
+
+def mingru_scan(zug: torch.Tensor, cu_seqlens: torch.Tensor, slot_ids: torch.Tensor, state: torch.Tensor,
+                out: torch.Tensor, chunks: Optional[torch.Tensor] = None) -> None:
+    """The minGRU recurrence over a ragged step.  `zug` float32 `[tokens][3 W]`: gate, candidate and
+    output-gate pre-activations; `state` float32 `[slots][W]`, read and left at each sequence's
+    last token for the rows `slot_ids`; `out` `[tokens][W]` (run type) = state * silu(g).  With
+    `chunks` (`scan_chunks`, on the device) the sequences are walked in chunks side by side."""
+    _need(zug, "mingru_scan.zug", torch.float32)
+    n_tok, w3 = zug.shape
+    if w3 % 3:
+        raise KernelError(f"mingru_scan: rows of {w3} values are not three equal parts")
+    w = w3 // 3
+    n_seqs = slot_ids.numel()
+    _need(cu_seqlens, "mingru_scan.cu_seqlens", torch.int32, (n_seqs + 1,))
+    _need(slot_ids, "mingru_scan.slot_ids", torch.int32, (n_seqs,))
+    _need(state, "mingru_scan.state", torch.float32)
+    if state.dim() != 2 or state.shape[1] != w:
+        raise KernelError(f"mingru_scan: state {tuple(state.shape)} for a width of {w}")
+    _need(out, "mingru_scan.out", _FLOATS, (n_tok, w))
+    if chunks is None:
+        _check(_fn("recurrence", "mf_mingru_scan")(_ptr(zug), _ptr(cu_seqlens), _ptr(slot_ids), _ptr(state), _ptr(out),
+                                                    _is_bf16(out), n_seqs, w, _stream()), "mingru_scan")
+        return
+    _need(chunks, "mingru_scan.chunks", torch.int32)
+    if chunks.dim() != 2 or chunks.shape[0] != 5:
+        raise KernelError(f"mingru_scan: chunk table {tuple(chunks.shape)}")
+    n_chunks = chunks.shape[1]
+    ws = workspace("scan", (2 * n_chunks + n_seqs) * w, zug.device)
+    _check(_fn("recurrence", "mf_mingru_scan_chunked")(
+        _ptr(zug), _ptr(chunks), n_chunks, _ptr(slot_ids), _ptr(state), _ptr(ws), c_void_p(ws.data_ptr() + 8 * n_chunks * w),
+        _ptr(out), _is_bf16(out), n_seqs, w, _stream()), "mingru_scan_chunked")
+
+
+# ------------------------------------------------------------------ latent attention
+def latent_prep(proj: torch.Tensor, off_dkv: int, off_gate: int, latent_weight: torch.Tensor, eps: float,
+                cos: torch.Tensor, sin: torch.Tensor, positions: torch.Tensor, seq_of_tok: torch.Tensor,
+                page_table: torch.Tensor, cache: torch.Tensor, q_plain: torch.Tensor, q_abs: torch.Tensor,
+                gate: torch.Tensor, n_heads: int, dim: int, rot_dim: int, rank: int, write_cache: bool = True) -> None:
+    """From the 32-bit rows [q | dkv | gates] of one product: the normed latent and the rotated
+    shared key part into the cache rows `[pages][64][rank + rot_dim]` at the tokens' positions, the
+    plain query parts into `q_plain` `[tokens][heads][dim]`, the rotated query parts into the last
+    `rot_dim` columns of `q_abs` `[tokens][heads][rank + rot_dim]`, sigmoid of the gates into `gate`.
+    The tables have one column per rotated pair (2i, 2i+1); values behind the pairs pass unchanged."""
+    n_tok = positions.numel()
+    ld = proj.shape[1]
+    dk = rank + rot_dim
+    _need(proj, "latent_prep.proj", torch.float32, (n_tok, ld))
+    if off_dkv < n_heads * (dim + rot_dim) or off_dkv + dk > ld or off_gate + n_heads > ld or off_gate < 0:
+        raise KernelError(f"latent_prep: offsets {off_dkv}, {off_gate} do not fit rows of {ld}")
+    _need(latent_weight, "latent_prep.latent_weight", torch.float32, (rank,))
+    _need(cos, "latent_prep.cos", torch.float32)
+    _need(sin, "latent_prep.sin", torch.float32, tuple(cos.shape))
+    rd = 2 * cos.shape[1]
+    if rd > rot_dim:
+        raise KernelError(f"latent_prep: {rd} rotated values in a part of {rot_dim}")
+    _need(positions, "latent_prep.positions", torch.int32, (n_tok,))
+    _need(seq_of_tok, "latent_prep.seq_of_tok", torch.int32, (n_tok,))
+    _need(page_table, "latent_prep.page_table", torch.int32)
+    _need(q_plain, "latent_prep.q_plain", _FLOATS, (n_tok, n_heads, dim))
+    _need(q_abs, "latent_prep.q_abs", q_plain.dtype, (n_tok, n_heads, dk))
+    _need(gate, "latent_prep.gate", torch.float32, (n_tok, n_heads))
+    _need(cache, "latent_prep.cache", q_plain.dtype)
+    if cache.dim() < 2 or cache.shape[-1] != dk or cache.numel() % (PAGE * dk):
+        raise KernelError(f"latent_prep: cache {tuple(cache.shape)} does not hold pages of {PAGE} rows of {dk}")
+    _check(_fn("attn_latent", "mf_latent_prep")(
+        _ptr(proj), ld, off_dkv, off_gate, _ptr(latent_weight), float(eps), _ptr(cos), _ptr(sin), rd, _ptr(positions),
+        _ptr(seq_of_tok), _ptr(page_table), page_table.shape[1], _ptr(cache), _ptr(q_plain), _ptr(q_abs), _ptr(gate),
+        _is_bf16(q_plain), n_tok, n_heads, dim, rot_dim, rank, 1 if write_cache else 0, _stream()), "latent_prep")
+
+
+def headwise_linear(x: torch.Tensor, n_in: int, wt: torch.Tensor, out: torch.Tensor, n_out: int,
+                    gate: Optional[torch.Tensor] = None) -> None:
+    """out[t][h][:n_out] = (gate[t][h] *) wt[h]^T x[t][h][:n_in] for `wt` `[heads][n_in][n_out]` (each
+    head's matrix stored input-major); x and out are `[tokens][heads][row]` with rows at least that
+    long, everything in the run type, sums in 32-bit."""
+    _need(x, "headwise_linear.x", _FLOATS)
+    if x.dim() != 3 or out.dim() != 3:
+        raise KernelError("headwise_linear: x and out are [tokens][heads][row]")
+    n_tok, heads, in_stride = x.shape
+    _need(wt, "headwise_linear.wt", x.dtype, (heads, n_in, n_out))
+    _need(out, "headwise_linear.out", x.dtype)
+    if tuple(out.shape[:2]) != (n_tok, heads) or out.shape[2] < n_out or in_stride < n_in:
+        raise KernelError(f"headwise_linear: x {tuple(x.shape)}, out {tuple(out.shape)}, matrix {tuple(wt.shape)}")
+    if n_in * 32 > 64 * 1024:
+        raise KernelError(f"headwise_linear: inputs of {n_in} values do not fit the kernel's staging")
+    if gate is not None:
+        _need(gate, "headwise_linear.gate", torch.float32, (n_tok, heads))
+    _check(_fn("attn_latent", "mf_headwise_linear")(_ptr(x), in_stride, _ptr(wt), _ptr(out), out.shape[2], _ptr(gate),
+                                                     _is_bf16(x), n_tok, heads, n_in, n_out, _stream()),
+           "headwise_linear")
+
+
+def latent_split_plan(n_tok: int, n_heads: int, max_len: int, target_blocks: Optional[int] = None) -> Tuple[int, int]:
+    """(n_splits, split_len) of the latent attention's keys: as many splits (whole pages, at most
+    64) as it takes to give every CU a block where the step's tokens alone do not."""
+    target = target_blocks or 2 * cu_count()
+    blocks = n_tok * ((n_heads + 3) // 4)
+    pages = (max_len + PAGE - 1) // PAGE
+    want = max(1, min(64, pages, target // max(1, blocks)))
+    per = (pages + want - 1) // want
+    return (pages + per - 1) // per, per * PAGE
+
+
+def latent_attn(q_abs: torch.Tensor, cache: torch.Tensor, page_table: torch.Tensor, positions: torch.Tensor,
+                seq_of_tok: torch.Tensor, out: torch.Tensor, rank: int, scale: float, window: int,
+                max_len: int) -> None:
+    """out[t][h][:] = sum_j softmax_j(scale q_abs[t][h] . row_j) row_j[:rank] over the cached rows
+    j <= position of the token's sequence (the last `window` of them when window > 0)."""
+    _need(q_abs, "latent_attn.q_abs", _FLOATS)
+    if q_abs.dim() != 3:
+        raise KernelError("latent_attn: q_abs is [tokens][heads][rank + rot_dim]")
+    n_tok, heads, dk = q_abs.shape
+    _need(cache, "latent_attn.cache", q_abs.dtype)
+    if cache.shape[-1] != dk or cache.numel() % (PAGE * dk) or not 0 < rank <= dk:
+        raise KernelError(f"latent_attn: cache {tuple(cache.shape)}, queries of {dk}, rank {rank}")
+    if rank > 1024 or (4 * dk + 4 * 256 + 4) * 4 > 64 * 1024:
+        raise KernelError(f"latent_attn: rank {rank} / row {dk} beyond what the kernel holds")
+    _need(out, "latent_attn.out", q_abs.dtype, (n_tok, heads, rank))
+    _need(page_table, "latent_attn.page_table", torch.int32)
+    _need(positions, "latent_attn.positions", torch.int32, (n_tok,))
+    _need(seq_of_tok, "latent_attn.seq_of_tok", torch.int32, (n_tok,))
+    if page_table.shape[1] * PAGE < max_len:
+        raise KernelError(f"latent_attn: page table of {page_table.shape[1]} columns for {max_len} positions")
+    n_splits, split_len = latent_split_plan(n_tok, heads, max_len)
+    part = workspace("latent_attn", n_tok * heads * n_splits * (rank + 2), q_abs.device) if n_splits > 1 else None
+    _check(_fn("attn_latent", "mf_latent_attn")(
+        _ptr(q_abs), _ptr(cache), _ptr(page_table), page_table.shape[1], _ptr(positions), _ptr(seq_of_tok), _ptr(out),
+        _ptr(part), _is_bf16(q_abs), n_tok, heads, rank, dk, float(scale), int(window), n_splits, split_len,
+        _stream()), "latent_attn")
 
 
 # ------------------------------------------------------------------ matrix products

@@ -4,7 +4,7 @@ from .base import (BLOCKS, EMBEDDINGS, FEED_FORWARDS, HEADS, MIXERS, NORMS, POSI
                    register_embedding, register_feed_forward, register_head, register_mixer, register_norm,
                    register_position)
 from .spec import BlockSpec, ModelSpec, PartSpec, RunEntry, straight_schedule
-from . import attention, block, embedding, feedforward, norm, rotary  # registers the built-in parts
+from . import attention, block, embedding, feedforward, latent_attention, norm, recurrent, rotary  # registers the built-in parts
 from .linear import Linear
 
 __all__ = ["BLOCKS", "EMBEDDINGS", "FEED_FORWARDS", "HEADS", "MIXERS", "NORMS", "POSITIONS", "Block", "Embedding",

@@ -67,6 +67,14 @@ class Norm(Part):
         weight vector, else None.  A product that follows such a norm may fold it in."""
         return None
 
+    def add_normed(self, y: torch.Tensor, h: torch.Tensor, cast_out: Optional[torch.Tensor] = None) -> None:
+        """h += norm(y), for arrangements that norm a branch's result before it joins the stream
+        (float32 rows both); `cast_out`, where given, also gets the new rows in bfloat16.  A norm
+        with a kernel for it does this in one launch."""
+        h.add_(self.forward(y).to(torch.float32))
+        if cast_out is not None:
+            cast_out.copy_(h)
+
 
 @dataclass
 class NormAhead:
@@ -151,15 +159,18 @@ class Mixer(Part):
         return None
 
     takes_normed = False     # True: `x` may arrive as a `Normed` (see there)
+    can_overwrite = False    # True: `forward(..., accumulate=False)` stores its output instead of adding it
 
     def forward(self, x: torch.Tensor, h: torch.Tensor, ctx, entry: int, writes_cache: bool) -> None:
         """Adds the mixer's output for the step's tokens into h.  `entry` is the cache entry
-        (`ctx.cache.kv(entry)` / `ctx.cache.state(entry)`)."""
+        (`ctx.cache.kv(entry)` / `ctx.cache.state(entry)`).  A mixer with `can_overwrite` also takes
+        `accumulate=False` and then stores its output into h, whatever h held."""
         raise NotImplementedError
 
 
 class FeedForward(Part):
     takes_normed = False     # True: `x` may arrive as a `Normed`
+    can_overwrite = False    # True: `forward(..., accumulate=False)` stores its output instead of adding it
 
     def forward(self, x: torch.Tensor, h: torch.Tensor, ctx) -> None:
         """Adds the feed-forward's output into h (h may hold fewer rows than the step)."""

@@ -1,4 +1,6 @@
-"""Pre-norm residual block: h += mixer(norm(h)); h += feed_forward(norm(h))
+"""Block arrangements.
+
+Pre-norm residual block: h += mixer(norm(h)); h += feed_forward(norm(h))
 (src/models/qwen2/graph.rs:59-177 of yusiwen/minfer).  When only some rows are wanted after
 this block (the last one of a step), they are gathered between the two halves, so the
 feed-forward runs on those rows only, as the reference does for its tail rows
@@ -48,4 +50,71 @@ class PreNormBlock(Block):
             announce_norm(ctx, after)
             self.feed_forward.forward(x, h, ctx)
             ctx.norm_next = None
+        return h
+
+
+@register_block("branch_norm")
+class BranchNormBlock(Block):
+    """h += N1(mixer(h)); h += N2(feed_forward(h)): the branches read the residual stream itself
+    (rounded to the run type) and only their results are normed, on the way into the stream.
+    norms: "mixer_out" behind the mixer, "feed_forward_out" behind the feed-forward; a block without
+    one branch has neither that branch nor its norm.
+
+    In bfloat16 the kernel that adds a normed result into the stream also leaves the new stream
+    rounded, which is the next branch's input (`ctx.stream_copy`), so no conversion runs between
+    the branches of a step."""
+
+    needs_mixer = False
+    needs_feed_forward = False
+    norm_names = ()
+    optional_norms = ("mixer_out", "feed_forward_out")
+
+    def __init__(self, mixer, feed_forward, norms, rt):
+        super().__init__(mixer, feed_forward, norms, rt)
+        for part, name in ((mixer, "mixer_out"), (feed_forward, "feed_forward_out")):
+            if (part is None) != (name not in self.norms):
+                raise ValueError(f"branch_norm block: a branch and the norm {name!r} behind it come together or not at all")
+
+    def _input(self, h, ctx):
+        """The stream in the run type: itself in 32-bit, else the rounded copy the last addition
+        left, or a conversion."""
+        if self.rt.dtype == torch.float32:
+            return h
+        kept = getattr(ctx, "stream_copy", None)
+        if kept is not None and kept[0] is h:
+            return kept[1]
+        x = torch.empty(h.shape, dtype=self.rt.dtype, device=h.device)
+        ops.convert(h, x)
+        return x
+
+    def _join(self, norm, y, h, ctx, want_copy: bool):
+        copy = None
+        if want_copy and self.rt.dtype == torch.bfloat16:
+            copy = torch.empty(h.shape, dtype=torch.bfloat16, device=h.device)
+        norm.add_normed(y, h, cast_out=copy)
+        ctx.stream_copy = None if copy is None else (h, copy)
+
+    @staticmethod
+    def _run(part, x, rows, width, *args):
+        """The branch's result as rows of their own (float32)."""
+        if getattr(part, "can_overwrite", False):
+            y = torch.empty((rows, width), dtype=torch.float32, device=x.device)
+            part.forward(x, y, *args, accumulate=False)
+        else:
+            y = torch.zeros((rows, width), dtype=torch.float32, device=x.device)
+            part.forward(x, y, *args)
+        return y
+
+    def forward(self, h, ctx, entry: int, writes_cache: bool, keep_rows=None):
+        ctx.norm_next = ctx.norm_ahead = None
+        if self.mixer is not None:
+            y = self._run(self.mixer, self._input(h, ctx), h.shape[0], h.shape[1], ctx, entry, writes_cache)
+            self._join(self.norms["mixer_out"], y, h, ctx, want_copy=keep_rows is None)
+        if keep_rows is not None:
+            kept = torch.empty((keep_rows.numel(), h.shape[1]), dtype=h.dtype, device=h.device)
+            ops.gather_rows(h, keep_rows, kept)
+            h = kept
+        if self.feed_forward is not None:
+            y = self._run(self.feed_forward, self._input(h, ctx), h.shape[0], h.shape[1], ctx)
+            self._join(self.norms["feed_forward_out"], y, h, ctx, want_copy=keep_rows is None)
         return h

@@ -9,7 +9,7 @@ import torch
 
 from ..kernels import ops
 from ..weights.loader import TensorSpec
-from .base import Embedding, Head, register_embedding, register_head
+from .base import NORMS, Runtime, Embedding, Head, make_part, register_embedding, register_head
 from .linear import Linear
 
 
@@ -34,6 +34,27 @@ class TokenEmbedding(Embedding):
 
     def forward(self, token_ids, out, ctx=None) -> None:
         ops.embed(self.weight, token_ids, out)
+
+
+@register_embedding("normed_token_embedding")
+class NormedTokenEmbedding(TokenEmbedding):
+    """The table's row, then a norm of its own over it before anything else reads the stream.
+    params: name (tensor), vocab_size, hidden_size, norm (PartSpec of a registered norm)."""
+
+    def __init__(self, spec, rt):
+        super().__init__(spec, rt)
+        self.norm = make_part(NORMS, spec.params["norm"], Runtime(torch.float32, rt.device), "norm")
+
+    def tensor_specs(self):
+        return dict(super().tensor_specs(), **self.norm.tensor_specs())
+
+    def load(self, get):
+        super().load(get)
+        self.norm.load(get)
+
+    def forward(self, token_ids, out, ctx=None) -> None:
+        ops.embed(self.weight, token_ids, out)
+        self.norm.forward(out, out=out)       # in place, 32-bit rows
 
 
 @register_head("linear_head")

@@ -68,3 +68,48 @@ class SwiGLU(FeedForward):
         else:
             ops.swiglu(self.gate_up(x, out_dtype=torch.float32), y)
         self.down(y, out=h, accumulate=True, ctx=ctx)
+
+
+def _softplus(v: float) -> float:
+    import math
+    return max(v, 0.0) + math.log1p(math.exp(-abs(v)))
+
+
+@register_feed_forward("dense_xielu")
+class DenseXIELU(FeedForward):
+    """down(act(up x + b_up)) + b_down with the xIELU activation: for z > 0, softplus(p) z^2 + z/2;
+    for z <= 0, (1/2 + softplus(q)) (e^z - 1 - z) + z/2, where (p, q) are the two values of the
+    layer's `act` tensor.  The activation reads the up product's 32-bit sums and is rounded once.
+    params: hidden_size, intermediate_size, up, down (tensor names; biases are name + ".b"), act."""
+
+    can_overwrite = True
+
+    def __init__(self, spec, rt):
+        super().__init__(spec, rt)
+        p = spec.params
+        self.hidden, self.inter = int(p["hidden_size"]), int(p["intermediate_size"])
+        self.names = {k: p[k] for k in ("up", "down", "act")}
+        self.up = self.down = None
+        self.a_pos = self.a_neg = None
+
+    def tensor_specs(self):
+        n = self.names
+        return {n["up"]: TensorSpec((self.inter, self.hidden)), n["up"] + ".b": TensorSpec((self.inter,)),
+                n["down"]: TensorSpec((self.hidden, self.inter)), n["down"] + ".b": TensorSpec((self.hidden,)),
+                n["act"]: TensorSpec((2,))}
+
+    def load(self, get):
+        n = self.names
+        self.up = Linear(get(n["up"]), get(n["up"] + ".b"))
+        self.down = Linear(get(n["down"]), get(n["down"] + ".b"))
+        pq = [float(v) for v in get(n["act"]).to(torch.float32).cpu()]
+        self.a_pos, self.a_neg = _softplus(pq[0]), 0.5 + _softplus(pq[1])
+
+    def decode_copies(self, make: bool, min_row_length: int = 0) -> int:
+        return self.up.decode_copy(make, min_row_length) + self.down.decode_copy(make, min_row_length)
+
+    def forward(self, x, h, ctx, accumulate: bool = True) -> None:
+        u = self.up(x, out_dtype=torch.float32)
+        y = torch.empty((x.shape[0], self.inter), dtype=self.rt.dtype, device=x.device)
+        ops.xielu(u, y, self.a_pos, self.a_neg)
+        self.down(y, out=h, accumulate=accumulate)

@@ -1,0 +1,100 @@
+"""Attention over a shared low-rank latent.
+
+Per token one latent c (rank values, RMS-normed with a weight of its own) and one rotated key
+part (rot_dim values) are computed and cached; head h's key is [Wuk_h c | k_rot] and its value
+Wuv_h c; the query of a head is [plain (dim) | rotated (rot_dim)]; scores are
+(q_plain . k_plain + q_rot . k_rot) * scale over the positions up to the token's own, ordinary
+softmax; a head's result is multiplied by sigmoid of a gate value computed from the mixer's
+input; the heads are concatenated and projected.
+
+The per-head keys and values are never built.  Wuk_h is applied to the query instead
+((Wuk_h^T q_plain) . c = q_plain . (Wuk_h c)) and Wuv_h to the attention's result over the cached
+latents, so the cache holds `rank + rot_dim` values a token whatever the number of heads, and a step's
+attention reads each cached row once for all heads.
+"""
+from __future__ import annotations
+
+import torch
+
+from ..cache.paged import KVRequest
+from ..kernels import ops
+from ..weights.loader import TensorSpec
+from .base import Mixer, POSITIONS, make_part, register_mixer
+from .linear import Linear
+
+
+@register_mixer("latent_attention")
+class LatentAttention(Mixer):
+    """params: hidden_size, n_heads, dim, rot_dim, v_dim, rank, scale, eps (of the latent's norm),
+    window (None or int), position (PartSpec of a pairwise rotation over at most rot_dim values),
+    q, dkv, dkv_norm, uk, uv, gate, o (tensor names)."""
+
+    can_overwrite = True
+
+    def __init__(self, spec, rt):
+        super().__init__(spec, rt)
+        p = spec.params
+        self.hidden, self.nh, self.dn, self.dr, self.dv, self.rank = (
+            int(p[k]) for k in ("hidden_size", "n_heads", "dim", "rot_dim", "v_dim", "rank"))
+        self.scale, self.eps = float(p["scale"]), float(p["eps"])
+        self.window = p.get("window")
+        if self.window is not None and int(self.window) < 1:
+            raise ValueError(f"latent_attention: window {self.window} must be >= 1")
+        self.names = {k: p[k] for k in ("q", "dkv", "dkv_norm", "uk", "uv", "gate", "o")}
+        self.position = make_part(POSITIONS, p["position"], rt, "position encoding")
+        if not hasattr(self.position, "pair_tables"):
+            raise ValueError("latent_attention: the position encoding must be a pairwise rotation (pair_tables)")
+        self.dk = self.rank + self.dr
+        self.proj = self.o = self.uk_t = self.uv_t = self.latent_weight = None
+
+    def tensor_specs(self):
+        n, H = self.names, self.nh
+        return {n["q"]: TensorSpec((H * (self.dn + self.dr), self.hidden)),
+                n["dkv"]: TensorSpec((self.dk, self.hidden)),
+                n["dkv_norm"]: TensorSpec((self.rank,), init="ones"),
+                n["uk"]: TensorSpec((H * self.dn, self.rank)),
+                n["uv"]: TensorSpec((H * self.dv, self.rank)),
+                n["gate"]: TensorSpec((H, self.hidden)),
+                n["o"]: TensorSpec((self.hidden, H * self.dv))}
+
+    def load(self, get):
+        n, H = self.names, self.nh
+        # q | dkv | gate over the same input: one product
+        self.proj = Linear.stacked([get(n["q"]), get(n["dkv"]), get(n["gate"])])
+        self.off_dkv = H * (self.dn + self.dr)
+        self.off_gate = self.off_dkv + self.dk
+        self.latent_weight = get(n["dkv_norm"]).to(torch.float32).contiguous()
+        # per-head matrices, input-major: uk_t[h] = Wuk_h [dim][rank] takes q_plain to the latent's
+        # side; uv_t[h] = Wuv_h^T [rank][v_dim] takes the result over the latents to the head's values
+        self.uk_t = get(n["uk"]).view(H, self.dn, self.rank).contiguous()
+        self.uv_t = get(n["uv"]).view(H, self.dv, self.rank).transpose(1, 2).contiguous()
+        self.o = Linear(get(n["o"]))
+
+    def cache_request(self):
+        # one shared "kv head" of rank + rot_dim values; the values are the rows' first `rank` columns
+        return KVRequest(1, self.dk, None if self.window is None else int(self.window), v_head_dim=0)
+
+    def decode_copies(self, make: bool, min_row_length: int = 0) -> int:
+        return self.proj.decode_copy(make, min_row_length) + self.o.decode_copy(make, min_row_length)
+
+    def prepare(self, max_len: int) -> None:
+        self.position.prepare(max_len)
+
+    def forward(self, x, h, ctx, entry: int, writes_cache: bool, accumulate: bool = True) -> None:
+        rows, _, group = ctx.cache.kv(entry)
+        table = ctx.page_table(group)
+        n, H, dev, dt = x.shape[0], self.nh, x.device, self.rt.dtype
+        proj = self.proj(x, out_dtype=torch.float32)
+        cos, sin = self.position.pair_tables(ctx.max_len)
+        q_plain = torch.empty((n, H, self.dn), dtype=dt, device=dev)
+        q_abs = torch.empty((n, H, self.dk), dtype=dt, device=dev)
+        gate = torch.empty((n, H), dtype=torch.float32, device=dev)
+        ops.latent_prep(proj, self.off_dkv, self.off_gate, self.latent_weight, self.eps, cos, sin, ctx.positions,
+                        ctx.seq_of_tok, table, rows, q_plain, q_abs, gate, H, self.dn, self.dr, self.rank, writes_cache)
+        ops.headwise_linear(q_plain, self.dn, self.uk_t, q_abs, self.rank)
+        o_lat = torch.empty((n, H, self.rank), dtype=dt, device=dev)
+        ops.latent_attn(q_abs, rows, table, ctx.positions, ctx.seq_of_tok, o_lat, self.rank, self.scale,
+                        0 if self.window is None else int(self.window), ctx.max_len)
+        o = torch.empty((n, H, self.dv), dtype=dt, device=dev)
+        ops.headwise_linear(o_lat, self.rank, self.uv_t, o, self.dv, gate=gate)
+        self.o(o.view(n, H * self.dv), out=h, accumulate=accumulate)

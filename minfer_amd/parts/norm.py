@@ -36,3 +36,39 @@ class RMSNorm(Norm):
             out = torch.empty((rows, self.size), dtype=self.rt.dtype, device=h.device)
         ops.rmsnorm(h, self.weight, self.eps, out, row_idx)
         return out
+
+
+@register_norm("group_rmsnorm")
+class GroupRMSNorm(Norm):
+    """RMS norm taken over `groups` equal consecutive parts of the vector: each part is divided by
+    its own sqrt(mean(part^2) + eps), then the whole is multiplied by the weight.  One group is the
+    plain RMS norm.  params: size, eps, groups, weight (tensor name)."""
+
+    def __init__(self, spec, rt):
+        super().__init__(spec, rt)
+        p = spec.params
+        self.size, self.eps, self.groups = int(p["size"]), float(p["eps"]), int(p.get("groups", 1))
+        self.name = p["weight"]
+        if self.groups < 1 or self.size % self.groups:
+            raise ValueError(f"group_rmsnorm: {self.size} values do not split into {self.groups} equal parts")
+        self.weight = None
+
+    def tensor_specs(self):
+        return {self.name: TensorSpec((self.size,), init="ones")}
+
+    def load(self, get):
+        self.weight = get(self.name).to(torch.float32).contiguous()
+
+    def rms_scale(self):
+        return (self.weight, self.eps) if self.groups == 1 else None
+
+    def forward(self, h, out: Optional[torch.Tensor] = None, row_idx: Optional[torch.Tensor] = None):
+        rows = h.shape[0] if row_idx is None else row_idx.numel()
+        if out is None:
+            out = torch.empty((rows, self.size), dtype=self.rt.dtype, device=h.device)
+        ops.group_rmsnorm(h, self.weight, self.eps, self.groups, out, row_idx)
+        return out
+
+    def add_normed(self, y, h, cast_out: Optional[torch.Tensor] = None) -> None:
+        """h += norm(y) in one kernel; `cast_out` (bfloat16) also gets the new rows rounded."""
+        ops.group_rmsnorm(y, self.weight, self.eps, self.groups, h, add=True, cast_out=cast_out)

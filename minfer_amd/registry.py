@@ -42,6 +42,8 @@ def load_config(folder_or_file: str):
 def _register_builtin() -> None:
     from .config.qwen2 import ARCHITECTURE, Qwen2Config
     register_architecture(ARCHITECTURE, Qwen2Config)
+    from .config import tabezen
+    register_architecture(tabezen.ARCHITECTURE, tabezen.TabezenConfig)
 
 
 _register_builtin()

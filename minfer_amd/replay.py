@@ -23,6 +23,10 @@ import sys
 
 import numpy as np
 
+from .cache.paged import PAGE
+
+SPARE_PAGES = 64      # pages beyond --max-tokens: each live request may leave most of its last page unused
+
 
 def parse_args(argv=None):
     ap = argparse.ArgumentParser(prog="trace_run", description=__doc__.split("\n\n")[0])
@@ -45,7 +49,8 @@ def run(args, stdin=None, stdout=None) -> int:
         torch.backends.cuda.matmul.allow_tf32 = False
     os.makedirs(args.out, exist_ok=True)
     model = load_model(args.model, dtype=args.dtype, device=args.device)
-    engine = Engine(model, max_tokens=max(64, args.max_tokens))
+    # every live request rounds up to whole pages: room for that on top of the tokens themselves
+    engine = Engine(model, max_tokens=max(64, args.max_tokens) + SPARE_PAGES * PAGE)
     slots = {}                                  # request id -> cache slot
     for line in stdin:
         line = line.strip()

@@ -202,6 +202,114 @@ def attn_prefill(q, kcache, vcache, page_table, ctx, out, n_heads, n_kv_heads, h
                 head_dim, scale, window, ctx.max_len)
 
 
+# ------------------------------------------------------------------ norm in groups, xIELU, pair rotation
+def group_rmsnorm(x, weight, eps, groups, out, row_idx=None, add=False, cast_out=None):
+    src = (x if row_idx is None else x[row_idx.long()]).double()
+    d = src.shape[-1]
+    parts = src.view(src.shape[0], groups, d // groups)
+    y = (parts / torch.sqrt((parts * parts).mean(dim=-1, keepdim=True) + eps)).reshape(src.shape)
+    if weight is not None:
+        y = y * weight.double()
+    if add:
+        y = y + out.double()
+    out.copy_(y.to(out.dtype))
+    if cast_out is not None:
+        cast_out.copy_(out.to(cast_out.dtype))
+
+
+def xielu(x, out, a_pos, a_neg):
+    z = x.double()
+    pos = a_pos * z * z + 0.5 * z
+    neg = a_neg * (torch.expm1(torch.clamp(z, max=0.0)) - z) + 0.5 * z
+    out.copy_(torch.where(z > 0, pos, neg).to(out.dtype))
+
+
+def rope_table_freqs(n_pos, freqs, magnitude, device):
+    f = torch.tensor([float(v) for v in freqs], dtype=torch.float64)
+    ang = torch.arange(n_pos, dtype=torch.float64)[:, None] * f[None, :]
+    return (torch.cos(ang) * magnitude).float().to(device), (torch.sin(ang) * magnitude).float().to(device)
+
+
+def _rotate_pairs(v, c, s):
+    """v [..., n]: the first 2 * c.shape[-1] values in pairs (2i, 2i+1); c, s broadcast over v's leading axes."""
+    rd = 2 * c.shape[-1]
+    out = v.clone()
+    a, b = v[..., 0:rd:2], v[..., 1:rd:2]
+    out[..., 0:rd:2] = a * c - b * s
+    out[..., 1:rd:2] = b * c + a * s
+    return out
+
+
+def rope_pairs_inplace(qkv, cos, sin, positions, n_rot_heads, n_heads_total, head_dim):
+    t = positions.numel()
+    x = qkv.double().view(t, n_heads_total, head_dim)
+    c, s = cos[positions.long()].double()[:, None, :], sin[positions.long()].double()[:, None, :]
+    x[:, :n_rot_heads] = _rotate_pairs(x[:, :n_rot_heads], c, s)
+    qkv.copy_(x.view(t, -1).to(qkv.dtype))
+
+
+# ------------------------------------------------------------------ recurrence
+def mingru_scan(zug, cu_seqlens, slot_ids, state, out, chunks=None):
+    w = zug.shape[1] // 3
+    z = torch.sigmoid(zug[:, :w].double())
+    u = zug[:, w:2 * w].double()
+    cand = torch.where(u >= 0, u + 0.5, torch.sigmoid(u))
+    g = zug[:, 2 * w:].double()
+    for b in range(slot_ids.numel()):
+        slot = int(slot_ids[b])
+        s = state[slot].double()
+        for t in range(int(cu_seqlens[b]), int(cu_seqlens[b + 1])):
+            s = (1.0 - z[t]) * s + z[t] * cand[t]
+            s = s.float().double()                       # the state is carried in 32-bit
+            out[t] = (s * g[t] * torch.sigmoid(g[t])).to(out.dtype)
+        state[slot] = s.float()
+
+
+# ------------------------------------------------------------------ latent attention
+def latent_prep(proj, off_dkv, off_gate, latent_weight, eps, cos, sin, positions, seq_of_tok, page_table, cache,
+                q_plain, q_abs, gate, n_heads, dim, rot_dim, rank, write_cache=True):
+    t = positions.numel()
+    p = proj.double()
+    c_t, s_t = cos[positions.long()].double(), sin[positions.long()].double()
+    q = p[:, :n_heads * (dim + rot_dim)].view(t, n_heads, dim + rot_dim)
+    q_plain.copy_(q[:, :, :dim].to(q_plain.dtype))
+    q_abs[:, :, rank:] = _rotate_pairs(q[:, :, dim:], c_t[:, None, :], s_t[:, None, :]).to(q_abs.dtype)
+    gate.copy_(torch.sigmoid(p[:, off_gate:off_gate + n_heads]).float())
+    if not write_cache:
+        return
+    c = p[:, off_dkv:off_dkv + rank]
+    c = c / torch.sqrt((c * c).mean(dim=-1, keepdim=True) + eps) * latent_weight.double()
+    k_rot = _rotate_pairs(p[:, off_dkv + rank:off_dkv + rank + rot_dim], c_t, s_t)
+    rows = torch.cat([c, k_rot], dim=-1).to(cache.dtype)
+    flat = cache.view(-1, PAGE, rank + rot_dim)
+    for i in range(t):
+        pos = int(positions[i])
+        page = int(page_table[int(seq_of_tok[i]), pos // PAGE])
+        assert page >= 0
+        flat[page, pos % PAGE] = rows[i]
+
+
+def headwise_linear(x, n_in, wt, out, n_out, gate=None):
+    y = torch.einsum("thi,hio->tho", x[:, :, :n_in].double(), wt.double())
+    if gate is not None:
+        y = y * gate.double()[:, :, None]
+    out[:, :, :n_out] = y.to(out.dtype)
+
+
+def latent_attn(q_abs, cache, page_table, positions, seq_of_tok, out, rank, scale, window, max_len):
+    t, heads, dk = q_abs.shape
+    flat = cache.view(-1, PAGE, dk)
+    for i in range(t):
+        p = int(positions[i])
+        lo = max(0, p - window + 1) if window else 0
+        pos = torch.arange(lo, p + 1)
+        page = page_table[int(seq_of_tok[i])].long()[pos // PAGE]
+        assert (page >= 0).all(), "attention reads a page that was given back"
+        rows = flat[page, pos % PAGE].double()           # [n][dk]
+        s = (q_abs[i].double() @ rows.t()) * scale       # [heads][n]
+        out[i] = (torch.softmax(s, dim=-1) @ rows[:, :rank]).to(out.dtype)
+
+
 # ------------------------------------------------------------------ sampling
 def argmax(logits, out):
     import plain_qwen2 as pq
@@ -271,7 +379,9 @@ def advance(next_ids, sampled, positions, steps, prev=None, n_prev=None, cursor=
 
 NAMES = ["embed", "rmsnorm", "gather_rows", "swiglu", "convert", "fill_normal", "rope_table",
          "rope_kvwrite", "rope_inplace", "linear", "attn_tokens", "attn_prefill", "argmax", "sample", "penalties",
-         "top_k", "top_p", "sample_filtered", "sample_filtered_takes", "advance", "interleave_gate_up", "linear_swiglu", "linear_normed", "linear_fused", "attn_decode_rope"]
+         "top_k", "top_p", "sample_filtered", "sample_filtered_takes", "advance", "interleave_gate_up", "linear_swiglu", "linear_normed", "linear_fused", "attn_decode_rope",
+         "group_rmsnorm", "xielu", "rope_table_freqs", "rope_pairs_inplace", "mingru_scan", "latent_prep",
+         "headwise_linear", "latent_attn"]
 
 
 def install(monkeypatch):
