@@ -68,6 +68,10 @@ def parse():
                     help="cache size in tokens (default: batch x context, or what fits in free memory if less)")
     ap.add_argument("--no-graph", action="store_true")
     ap.add_argument("--only", choices=["decode", "prefill"], help="run one part (for profiles); prints no JSON line")
+    ap.add_argument("--design", choices=["tabezen"], default=None,
+                    help="instead of the default workload: prefill and decode of this design at a few layer sizes "
+                         "beside the Qwen2 decoder of the same width, depth and feed-forward size, kernel by kernel")
+    ap.add_argument("--design-sizes", default="small,medium", help="which of the design's sizes to run")
     return ap.parse_args()
 
 
@@ -96,6 +100,10 @@ def prefill_flops(cfg, t):
     gemm = 2.0 * t * L * per_layer + 2.0 * head          # the head runs on the one wanted row
     attn = L * 2.0 * nh * hd * t * (t + 1)               # causal: QK^T and PV over t(t+1)/2 pairs
     return gemm + attn
+
+
+def vocab_of(cfg):
+    return cfg["vocab_size"] if "vocab_size" in cfg else cfg["vocab"]
 
 
 def prompt_lengths(batch, prompt_max, seed=0):
@@ -146,8 +154,8 @@ def kernel_breakdown(eng, cfg, batch, prompt_max):
     lens = prompt_lengths(batch, prompt_max)
     slots = [eng.new_sequence() for _ in lens]
     for s, n in zip(slots, lens):
-        eng.step([s], [[int(t) for t in rng.integers(0, cfg["vocab_size"], size=n)]], [[]])
-    toks = [[int(t)] for t in rng.integers(0, cfg["vocab_size"], size=batch)]
+        eng.step([s], [[int(t) for t in rng.integers(0, vocab_of(cfg), size=n)]], [[]])
+    toks = [[int(t)] for t in rng.integers(0, vocab_of(cfg), size=batch)]
     eng.step(slots, toks, "last")                       # warm: tables, workspaces
     ctx = eng.build_context(slots, toks, "last")        # (its upload waits for the stream, so it comes first)
     torch.cuda.synchronize()
@@ -165,14 +173,14 @@ def kernel_breakdown(eng, cfg, batch, prompt_max):
     return sorted(((k, n, t) for k, (n, t) in agg.items()), key=lambda r: -r[2])
 
 
-def run_decode(eng, cfg, batch, prompt_max, steps, warmup, use_graph, elem, seed=0):
+def run_decode(eng, cfg, batch, prompt_max, steps, warmup, use_graph, elem, seed=0, bytes_fn=None):
     """Prefills `batch` unequal prompts (untimed), then times `steps` decode steps."""
     import numpy as np
     import torch
     from minfer_amd.sampling import Sampler, SamplingParams
     rng = np.random.default_rng(1)
     lens = prompt_lengths(batch, prompt_max, seed)
-    prompts = [[int(t) for t in rng.integers(0, cfg["vocab_size"], size=n)] for n in lens]
+    prompts = [[int(t) for t in rng.integers(0, vocab_of(cfg), size=n)] for n in lens]
     slots = [eng.new_sequence() for _ in prompts]
     first, group, toks = [], [], 0
     for i, p in enumerate(prompts):            # prompts in steps of at most 8192 tokens
@@ -206,7 +214,7 @@ def run_decode(eng, cfg, batch, prompt_max, steps, warmup, use_graph, elem, seed
     ctx_end = sum(eng.length(s) for s in slots)
     for s in slots:
         eng.end_sequence(s)
-    nbytes = decode_bytes(cfg, elem, (ctx_start + ctx_end) / 2.0)
+    nbytes = (bytes_fn or decode_bytes)(cfg, elem, (ctx_start + ctx_end) / 2.0)
     return dict(tok_s=batch * steps / dt, ms=dt / steps * 1e3, gbs=nbytes / (dt / steps) / 1e9, bytes=nbytes)
 
 
@@ -214,7 +222,7 @@ def run_prefill(eng, cfg, n_tokens, repeats=5):
     import numpy as np
     import torch
     rng = np.random.default_rng(2)
-    prompt = [int(t) for t in rng.integers(0, cfg["vocab_size"], size=n_tokens)]
+    prompt = [int(t) for t in rng.integers(0, vocab_of(cfg), size=n_tokens)]
     times = []
     for i in range(repeats + 2):
         s = eng.new_sequence()
@@ -228,11 +236,128 @@ def run_prefill(eng, cfg, n_tokens, repeats=5):
     return statistics.median(times)
 
 
+# ---------------------------------------------------------------- another design beside the default one
+def tabezen_config(width, layers, heads, ff, rank=512, dim=128, rot_dim=64, vdim=128, gru_width=None, vocab=32768):
+    """Attention over a latent of `rank` values and minGRU layers in turn, each with a dense feed-forward."""
+    att = dict(type="latent_attention",
+               mixer=dict(heads=heads, dim=dim, rot_dim=rot_dim, vdim=vdim, kv_rank=rank, scale=(dim + rot_dim) ** -0.5,
+                          rot=dict(base=10000.0, dims=rot_dim,
+                                   scaling=dict(factor=8.0, original=4096, fast=32.0, slow=1.0))),
+               mlp=dict(kind="dense", ff=ff))
+    gru = dict(type="mingru", mixer=dict(width=gru_width or width), mlp=dict(kind="dense", ff=ff))
+    return dict(architecture="Tabezen", vocab=vocab, width=width, norm=dict(eps=1e-6, groups=4),
+                layers=[att if i % 2 == 0 else gru for i in range(layers)])
+
+
+def qwen2_like(width, layers, heads, ff, vocab=32768):
+    """The Qwen2 decoder of the same width, depth, head count and feed-forward size (head size 128)."""
+    return dict(QWEN25_7B, num_hidden_layers=layers, hidden_size=width, num_attention_heads=heads,
+                num_key_value_heads=max(1, heads // 4), head_dim=128, intermediate_size=ff, vocab_size=vocab,
+                max_position_embeddings=8192)
+
+
+DESIGN_SIZES = {
+    "small": dict(width=2048, layers=4, heads=16, ff=8192),
+    "medium": dict(width=4096, layers=4, heads=32, ff=14336),
+}
+
+
+def traced_step(eng, slots, toks, want):
+    """One eager step with an event behind every launch: [(launch name, calls, microseconds)]."""
+    import torch
+    from minfer_amd.kernels import ops
+    ctx = eng.build_context(slots, toks, want)
+    torch.cuda.synchronize()
+    ops.probe_mfma(200000)
+    ops.start_trace()
+    eng.model.forward(ctx)
+    rows = ops.stop_trace()
+    eng.cache.commit(ctx.new_lengths)
+    agg = {}
+    for name, us in rows:
+        n, t = agg.get(name, (0, 0.0))
+        agg[name] = (n + 1, t + us)
+    return {k: dict(calls=n, us=round(t, 1)) for k, (n, t) in sorted(agg.items(), key=lambda r: -r[1][1])}
+
+
+def design_point(cfg, a, dtype, elem):
+    """Prefill of --prefill-tokens and decode at --batch for one configuration, with both steps' kernels."""
+    import numpy as np
+    import torch
+    from minfer_amd import LLM
+    llm = LLM(config=cfg, random_weights=True, weight_seed=0, dtype=dtype, n_ctx=a.context, n_slots=a.batch)
+    eng = llm.engine
+    rng = np.random.default_rng(5)
+    pre_s = run_prefill(eng, cfg, a.prefill_tokens, repeats=3)
+    s = eng.new_sequence()
+    pre_kernels = traced_step(eng, [s], [[int(t) for t in rng.integers(0, vocab_of(cfg), size=a.prefill_tokens)]], "last")
+    eng.end_sequence(s)
+    dec = run_decode(eng, cfg, a.batch, a.prompt_max, a.steps, a.warmup, not a.no_graph, elem, bytes_fn=lambda *_: 0.0)
+    slots = [eng.new_sequence() for _ in range(a.batch)]
+    for sl, n in zip(slots, prompt_lengths(a.batch, a.prompt_max)):
+        eng.step([sl], [[int(t) for t in rng.integers(0, vocab_of(cfg), size=n)]], [[]])
+    toks = [[int(t)] for t in rng.integers(0, vocab_of(cfg), size=a.batch)]
+    eng.step(slots, toks, "last")
+    dec_kernels = traced_step(eng, slots, toks, "last")
+    for sl in slots:
+        eng.end_sequence(sl)
+    out = dict(prefill_ms=round(pre_s * 1e3, 3), prefill_tok_s=round(a.prefill_tokens / pre_s, 1),
+               decode_ms=round(dec["ms"], 4), decode_tok_s=round(dec["tok_s"], 1),
+               prefill_kernels=pre_kernels, decode_kernels=dec_kernels)
+    del eng, llm
+    gc.collect()
+    torch.cuda.empty_cache()
+    return out
+
+
+def attention_rooflines(size, a, point, design):
+    """Fractions of the matrix cores' peak (prompt attention) and of the memory's (decode attention)
+    that the attention kernels of a measured point reach."""
+    t, L = a.prefill_tokens, size["layers"]
+    mean_ctx = sum(prompt_lengths(a.batch, a.prompt_max)) / a.batch
+    pk, dk = point["prefill_kernels"], point["decode_kernels"]
+    if design:
+        n_att = (L + 1) // 2
+        rank, row = 512, 576
+        flops = 2.0 * size["heads"] * (row + rank) * t * (t + 1) / 2 * n_att
+        pre_us = sum(v["us"] for k, v in pk.items() if k.startswith("latent_attn"))
+        nbytes = a.batch * mean_ctx * row * 2 * n_att
+        dec_us = sum(v["us"] for k, v in dk.items() if k.startswith("latent_attn"))
+    else:
+        flops = 2.0 * size["heads"] * 2 * 128 * t * (t + 1) / 2 * L
+        pre_us = sum(v["us"] for k, v in pk.items() if k.startswith("attn_prefill"))
+        nbytes = a.batch * mean_ctx * max(1, size["heads"] // 4) * 2 * 128 * 2 * L
+        dec_us = sum(v["us"] for k, v in dk.items() if k.startswith("attn_decode"))
+    return dict(prefill_attention_us=round(pre_us, 1),
+                prefill_attention_of_peak=round(flops / (pre_us * 1e-6) / PEAK_FLOPS["bf16"], 4) if pre_us else None,
+                decode_attention_us=round(dec_us, 1),
+                decode_attention_of_hbm=round(nbytes / (dec_us * 1e-6) / 1e9 / HBM_GBS, 4) if dec_us else None)
+
+
+def run_design(a) -> int:
+    dtype = {"bf16": "bfloat16", "fp32": "float32"}[a.dtype]
+    elem = 2 if a.dtype == "bf16" else 4
+    out = {"design": a.design, "dtype": a.dtype, "data": "synthetic", "batch": a.batch, "prompt_max": a.prompt_max,
+           "prefill_tokens": a.prefill_tokens, "steps": a.steps, "warmup": a.warmup, "sizes": {}}
+    for name in a.design_sizes.split(","):
+        size = DESIGN_SIZES[name]
+        row = {"size": size}
+        for label, cfg in (("tabezen", tabezen_config(**size)), ("qwen2", qwen2_like(**size))):
+            print(f"{name}: {label} ...", file=sys.stderr, flush=True)
+            row[label] = design_point(cfg, a, dtype, elem)
+            row[label]["attention"] = attention_rooflines(size, a, row[label], label == "tabezen")
+        out["sizes"][name] = row
+    print(json.dumps(out))
+    return 0
+
+
 def main() -> int:
     a = parse()
     if a.gpus != 1:
         print(f"bench.py measures one GPU; --gpus {a.gpus} is not supported (this engine runs on a single MI355X)")
         return 2
+    if a.design:
+        return run_design(a)
     import torch
     from minfer_amd import LLM, Engine
     shape_name, shape = SHAPES[a.shape]

@@ -31,10 +31,13 @@ LIBRARIES: Dict[str, str] = {
     "attn_decode_bf16": "attn_decode_bf16.hip",
     "attn_prefill_bf16": "attn_prefill_bf16.hip",
     "attn_latent": "attn_latent.hip",
+    "attn_latent_mfma": "attn_latent_mfma.hip",
     "recurrence": "recurrence.hip",
     "sampling": "sampling.hip",
     "probe": "probe.hip",
 }
+# library name -> extra -D definitions (variants of one source compiled for given sizes, see `variant`)
+DEFINES: Dict[str, List[str]] = {}
 HEADERS = {"host_random": ["random_normal.h"],
            "elementwise": ["common.h", "random_normal.h"],
            "attn_tokens_f32": ["common.h", "attn_tokens_impl.h"],
@@ -48,6 +51,19 @@ HOST_FLAGS = ["-O2", "-std=c++17", "-fPIC", "-shared", "-pthread", "-ffp-contrac
 
 class KernelBuildError(RuntimeError):
     pass
+
+
+def variant(base: str, **sizes: int) -> str:
+    """Registers (once) and names the library that is `base`'s source compiled with the given
+    sizes as definitions (`-DNAME=value`): kernels whose tiles and register arrays depend on a
+    model's sizes are built for the sizes at hand the first time a model with them runs."""
+    name = base + "".join(f"_{k.lower()}{int(v)}" for k, v in sorted(sizes.items()))
+    if name not in LIBRARIES:
+        LIBRARIES[name] = LIBRARIES[base]
+        DEFINES[name] = DEFINES.get(base, []) + [f"-D{k}={int(v)}" for k, v in sorted(sizes.items())]
+        if base in HEADERS:
+            HEADERS[name] = HEADERS[base]
+    return name
 
 
 def _hipcc() -> str:
@@ -71,7 +87,7 @@ def _host_compiler() -> str:
 
 def source_hash(name: str) -> str:
     h = hashlib.sha256()
-    h.update(" ".join(HOST_FLAGS if is_host_library(name) else HIPCC_FLAGS).encode())
+    h.update(" ".join((HOST_FLAGS if is_host_library(name) else HIPCC_FLAGS) + DEFINES.get(name, [])).encode())
     for fname in [LIBRARIES[name]] + HEADERS.get(name, ["common.h"]):
         with open(os.path.join(CSRC, fname), "rb") as f:
             h.update(fname.encode())
@@ -124,7 +140,7 @@ def compile_library(name: str, quiet: bool = False) -> str:
     if is_host_library(name):
         cmd = [_host_compiler()] + HOST_FLAGS + ["-I", CSRC, os.path.join(CSRC, LIBRARIES[name]), "-o", tmp]
     else:
-        cmd = [_hipcc()] + HIPCC_FLAGS + ["-I", CSRC, os.path.join(CSRC, LIBRARIES[name]), "-o", tmp]
+        cmd = [_hipcc()] + HIPCC_FLAGS + DEFINES.get(name, []) + ["-I", CSRC, os.path.join(CSRC, LIBRARIES[name]), "-o", tmp]
     if not quiet:
         _say(f"compiling {LIBRARIES[name]}" + ("" if is_host_library(name) else " for gfx950") + " ...")
     t0 = time.time()

@@ -56,6 +56,10 @@ _PROTOTYPES = {
         "mf_latent_attn": [_P, _P, _P, c_int, _P, _P, _P, _P, c_int, c_int, c_int, c_int, c_int, c_float, c_int,
                            c_int, c_int, _P],
     },
+    "attn_latent_mfma": {
+        "mf_latent_mfma": [_P, _P, _P, c_int, _P, _P, _P, _P, c_int, _P, _P, c_int, c_int, c_int, c_int, c_int, c_int,
+                           c_float, c_int, c_int, c_int, _P],
+    },
     "probe": {
         "mf_probe_read": [_P, c_size_t, _P, c_int, _P],
         "mf_probe_mfma": [c_int, _P, c_int, _P],
@@ -109,13 +113,16 @@ _PROTOTYPES = {
 _functions: Dict[str, object] = {}
 
 
-def _fn(lib: str, name: str):
-    f = _functions.get(name)
+def _fn(lib: str, name: str, variant: Optional[str] = None):
+    """`variant`: the name of a sized variant of `lib` (`build.variant`), whose functions have the
+    prototypes of `lib`."""
+    key = name if variant is None else f"{variant}:{name}"
+    f = _functions.get(key)
     if f is None:
-        f = getattr(build.load(lib), name)
+        f = getattr(build.load(variant or lib), name)
         f.argtypes = _PROTOTYPES[lib][name]
         f.restype = c_int
-        _functions[name] = f
+        _functions[key] = f
     return f
 
 
@@ -599,22 +606,35 @@ def headwise_linear(x: torch.Tensor, n_in: int, wt: torch.Tensor, out: torch.Ten
            "headwise_linear")
 
 
-def latent_split_plan(n_tok: int, n_heads: int, max_len: int, target_blocks: Optional[int] = None) -> Tuple[int, int]:
+def latent_split_plan(n_blocks: int, max_len: int, target_blocks: Optional[int] = None) -> Tuple[int, int]:
     """(n_splits, split_len) of the latent attention's keys: as many splits (whole pages, at most
-    64) as it takes to give every CU a block where the step's tokens alone do not."""
+    64) as it takes to give every CU a block where the step's `n_blocks` alone do not."""
     target = target_blocks or 2 * cu_count()
-    blocks = n_tok * ((n_heads + 3) // 4)
     pages = (max_len + PAGE - 1) // PAGE
-    want = max(1, min(64, pages, target // max(1, blocks)))
+    want = max(1, min(64, pages, target // max(1, n_blocks)))
     per = (pages + want - 1) // want
     return (pages + per - 1) // per, per * PAGE
 
 
+LATENT_MFMA_ROWS = 64        # (token, head) rows of a workgroup of the matrix-core latent attention
+LATENT_MFMA_MAX = (640, 512)  # padded row and rank up to which its registers hold queries and accumulators
+
+
+def latent_mfma_takes(dtype, rank: int, dk: int) -> bool:
+    """Whether the matrix-core kernel is built for these sizes: bfloat16, rows and rank multiples
+    of 8 (16-byte pieces), padded sizes within what a wave's registers hold."""
+    pad = lambda v: (v + 31) // 32 * 32
+    return (dtype == torch.bfloat16 and rank % 8 == 0 and dk % 8 == 0 and pad(dk) <= LATENT_MFMA_MAX[0]
+            and pad(rank) <= LATENT_MFMA_MAX[1] and not tuning.NO_LATENT_MFMA)
+
+
 def latent_attn(q_abs: torch.Tensor, cache: torch.Tensor, page_table: torch.Tensor, positions: torch.Tensor,
                 seq_of_tok: torch.Tensor, out: torch.Tensor, rank: int, scale: float, window: int,
-                max_len: int) -> None:
+                max_len: int, ctx=None) -> None:
     """out[t][h][:] = sum_j softmax_j(scale q_abs[t][h] . row_j) row_j[:rank] over the cached rows
-    j <= position of the token's sequence (the last `window` of them when window > 0)."""
+    j <= position of the token's sequence (the last `window` of them when window > 0).  With the
+    step's context (`ctx`: its ragged layout) and sizes the matrix-core kernel is built for, that
+    kernel runs: a workgroup per 64 (token, head) rows that share their keys."""
     _need(q_abs, "latent_attn.q_abs", _FLOATS)
     if q_abs.dim() != 3:
         raise KernelError("latent_attn: q_abs is [tokens][heads][rank + rot_dim]")
@@ -622,15 +642,33 @@ def latent_attn(q_abs: torch.Tensor, cache: torch.Tensor, page_table: torch.Tens
     _need(cache, "latent_attn.cache", q_abs.dtype)
     if cache.shape[-1] != dk or cache.numel() % (PAGE * dk) or not 0 < rank <= dk:
         raise KernelError(f"latent_attn: cache {tuple(cache.shape)}, queries of {dk}, rank {rank}")
-    if rank > 1024 or (4 * dk + 4 * 256 + 4) * 4 > 64 * 1024:
-        raise KernelError(f"latent_attn: rank {rank} / row {dk} beyond what the kernel holds")
     _need(out, "latent_attn.out", q_abs.dtype, (n_tok, heads, rank))
     _need(page_table, "latent_attn.page_table", torch.int32)
     _need(positions, "latent_attn.positions", torch.int32, (n_tok,))
     _need(seq_of_tok, "latent_attn.seq_of_tok", torch.int32, (n_tok,))
     if page_table.shape[1] * PAGE < max_len:
         raise KernelError(f"latent_attn: page table of {page_table.shape[1]} columns for {max_len} positions")
-    n_splits, split_len = latent_split_plan(n_tok, heads, max_len)
+    if ctx is not None and latent_mfma_takes(q_abs.dtype, rank, dk):
+        hc = min(heads, LATENT_MFMA_ROWS)
+        tq = LATENT_MFMA_ROWS // hc
+        if ctx.all_decode:
+            tile_seq = tile_q0 = None
+            n_tiles = n_tok
+        else:
+            tile_seq, tile_q0 = ctx.query_tiles(tq)
+            n_tiles = tile_seq.numel()
+        _need(ctx.cu_seqlens, "latent_attn.cu_seqlens", torch.int32, (page_table.shape[0] + 1,))
+        n_splits, split_len = latent_split_plan(n_tiles * ((heads + hc - 1) // hc), max_len)
+        part = workspace("latent_attn", n_tok * heads * n_splits * (rank + 2), q_abs.device) if n_splits > 1 else None
+        lib = build.variant("attn_latent_mfma", MF_LAT_DKP=(dk + 31) // 32 * 32, MF_LAT_RP=(rank + 31) // 32 * 32)
+        _check(_fn("attn_latent_mfma", "mf_latent_mfma", lib)(
+            _ptr(q_abs), _ptr(cache), _ptr(page_table), page_table.shape[1], _ptr(positions), _ptr(ctx.cu_seqlens),
+            _ptr(tile_seq), _ptr(tile_q0), n_tiles, _ptr(out), _ptr(part), n_tok, heads, rank, dk, hc, tq, float(scale),
+            int(window), n_splits, split_len, _stream()), "latent_attn_mfma")
+        return
+    if rank > 1024 or (4 * dk + 4 * 256 + 4) * 4 > 64 * 1024:
+        raise KernelError(f"latent_attn: rank {rank} / row {dk} beyond what the kernel holds")
+    n_splits, split_len = latent_split_plan(n_tok * ((heads + 3) // 4), max_len)
     part = workspace("latent_attn", n_tok * heads * n_splits * (rank + 2), q_abs.device) if n_splits > 1 else None
     _check(_fn("attn_latent", "mf_latent_attn")(
         _ptr(q_abs), _ptr(cache), _ptr(page_table), page_table.shape[1], _ptr(positions), _ptr(seq_of_tok), _ptr(out),

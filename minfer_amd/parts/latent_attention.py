@@ -94,7 +94,7 @@ class LatentAttention(Mixer):
         ops.headwise_linear(q_plain, self.dn, self.uk_t, q_abs, self.rank)
         o_lat = torch.empty((n, H, self.rank), dtype=dt, device=dev)
         ops.latent_attn(q_abs, rows, table, ctx.positions, ctx.seq_of_tok, o_lat, self.rank, self.scale,
-                        0 if self.window is None else int(self.window), ctx.max_len)
+                        0 if self.window is None else int(self.window), ctx.max_len, ctx=ctx)
         o = torch.empty((n, H, self.dv), dtype=dt, device=dev)
         ops.headwise_linear(o_lat, self.rank, self.uv_t, o, self.dv, gate=gate)
         self.o(o.view(n, H * self.dv), out=h, accumulate=accumulate)

@@ -296,7 +296,7 @@ def headwise_linear(x, n_in, wt, out, n_out, gate=None):
     out[:, :, :n_out] = y.to(out.dtype)
 
 
-def latent_attn(q_abs, cache, page_table, positions, seq_of_tok, out, rank, scale, window, max_len):
+def latent_attn(q_abs, cache, page_table, positions, seq_of_tok, out, rank, scale, window, max_len, ctx=None):
     t, heads, dk = q_abs.shape
     flat = cache.view(-1, PAGE, dk)
     for i in range(t):

@@ -205,6 +205,53 @@ def test_latent_attention_kernel_far_keys_and_page_edges(dtype, heads, rank, rot
                     assert (got[i].cpu().float() - row[None, :]).abs().max() < 0.15 * row.abs().max()
 
 
+def _step_context(lens, new, table):
+    """The ragged layout of a step in which sequence b (of lens[b] tokens) brings its last new[b]."""
+    from minfer_amd.engine.batch import StepContext
+    start = [n - k for n, k in zip(lens, new)]
+    seq = torch.repeat_interleave(torch.arange(len(lens)), torch.tensor(new)).int()
+    pos = torch.cat([torch.arange(s, s + k) for s, k in zip(start, new)]).int()
+    cu = torch.tensor([0] + list(np.cumsum(new)), dtype=torch.int32)
+    return StepContext(cache=None, n_tokens=sum(new), n_seqs=len(lens), token_ids=torch.zeros(sum(new), dtype=torch.int32, device=DEV),
+                       positions=pos.to(DEV), seq_of_tok=seq.to(DEV), cu_seqlens=cu.to(DEV),
+                       start_pos=torch.tensor(start, dtype=torch.int32, device=DEV),
+                       slot_ids=torch.arange(len(lens), dtype=torch.int32, device=DEV), logit_rows=None,
+                       page_tables={0: table.to(DEV)}, max_len=max(lens), max_new=max(new),
+                       all_decode=all(k == 1 for k in new), host_new=list(new), host_start=start), seq, pos
+
+
+@pytest.mark.parametrize("heads, rank, rot, window", [(3, 40, 8, 0), (5, 72, 16, 0), (2, 264, 8, 0), (1, 24, 16, 70),
+                                                      (16, 64, 32, 0), (70, 32, 8, 0)])
+@pytest.mark.parametrize("new", [(1, 64, 65, 700, 130), (1, 1, 1, 1, 1), (1, 2, 40, 33, 129)])
+def test_latent_attention_matrix_core_kernel(heads, rank, rot, window, new):
+    """The matrix-core kernel on ragged steps (whole prompts, one token each, portions on top of
+    a context) over shuffled pages of a NaN-poisoned pool, with and without a row that decides."""
+    from minfer_amd.kernels import ops
+    lens = (1, 64, 65, 700, 130)
+    assert ops.latent_mfma_takes(torch.bfloat16, rank, rank + rot)
+    for needle in (None, (3, 5), (3, 64), (4, 127)):
+        if window and needle:
+            continue
+        cache, table, _, _, _ = _latent_case(torch.bfloat16, heads, rank, rot, lens, seed=13, needle=needle)
+        ctx, seq, pos = _step_context(lens, new, table)
+        q = rnd(len(seq), heads, rank + rot, seed=60, scale=0.5)
+        if needle:
+            b, p = needle
+            row = cache.view(-1, 64, rank + rot)[table[b, p // 64], p % 64].float()
+            for i in range(len(seq)):
+                if seq[i] == b:
+                    q[i] = row[None, :] * 0.5 + 0.05 * q[i]
+        q = q.to(torch.bfloat16)
+        want = torch.empty(len(seq), heads, rank, dtype=torch.bfloat16)
+        plain_ops.latent_attn(q, cache, table, pos, seq, want, rank, 0.35, window, max(lens))
+        got = torch.full((len(seq), heads, rank), float("nan"), dtype=torch.bfloat16, device=DEV)
+        ops.latent_attn(q.to(DEV), cache.to(DEV), table.to(DEV), pos.to(DEV), seq.to(DEV), got, rank, 0.35, window,
+                        max(lens), ctx=ctx)
+        assert torch.isfinite(got).all()
+        err = (got.cpu().float() - want.float()).abs().max()
+        assert err < 4e-2, f"needle {needle}: {err}"
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_latent_prep_kernel(dtype):
     from minfer_amd.kernels import ops
