@@ -122,7 +122,7 @@ __global__ __launch_bounds__(256) void headwise_linear_kernel(const T* __restric
   }
   __syncthreads();
   const T* w = wt + (size_t)h * NI * NO;
-  for (int o = threadIdx.x; o < NO; o += 256) {
+  for (int o = blockIdx.z * 256 + threadIdx.x; o < NO; o += 256 * gridDim.z) {
     float acc[MF_HW_TT];
 #pragma unroll
     for (int tt = 0; tt < MF_HW_TT; ++tt) acc[tt] = 0.f;
@@ -146,13 +146,91 @@ MF_API int mf_headwise_linear(const void* in, int in_stride, const void* wt, voi
   if (n_tok <= 0) return 0;
   const size_t lds = (size_t)MF_HW_TT * NI * sizeof(float);
   if (H < 1 || NI < 1 || NO < 1 || lds > 64 * 1024) return (int)hipErrorInvalidValue;
-  dim3 grid((n_tok + MF_HW_TT - 1) / MF_HW_TT, H);
+  dim3 grid((n_tok + MF_HW_TT - 1) / MF_HW_TT, H, (NO + 255) / 256);
   if (is_bf16)
     headwise_linear_kernel<bf16><<<grid, 256, lds, stream>>>((const bf16*)in, in_stride, (const bf16*)wt, (bf16*)out,
                                                               out_stride, gate, n_tok, H, NI, NO);
   else
     headwise_linear_kernel<float><<<grid, 256, lds, stream>>>((const float*)in, in_stride, (const float*)wt,
                                                                (float*)out, out_stride, gate, n_tok, H, NI, NO);
+  return mf_launch_status();
+}
+
+// The same on the matrix cores (bfloat16, NI a multiple of 8): `wo` holds each head's matrix
+// output-major ([NO][NI]).  A wave takes 16 tokens x 64 outputs of one head and forms
+// D^T = W X^T with 16x16x32 MFMA, operands straight from memory (a lane's 8 consecutive inputs are
+// 16 bytes of a row in both), so that a lane ends up with four neighbouring outputs of one token.
+// Tasks are numbered head, output tile, token tile (fastest): the four waves of a block share a
+// head's rows of W where the step has tokens enough, and spread over the outputs where not.
+typedef unsigned int hw_u32x4 __attribute__((ext_vector_type(4)));
+
+__global__ __launch_bounds__(256) void headwise_mfma_kernel(const bf16* __restrict__ in, int in_stride,
+                                                            const bf16* __restrict__ wo, bf16* __restrict__ out,
+                                                            int out_stride, const float* __restrict__ gate, int n_tok,
+                                                            int H, int NI, int NO, int n_ttiles, int n_otiles) {
+  const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+  const int task = blockIdx.x * 4 + wv;
+  if (task >= H * n_otiles * n_ttiles) return;
+  const int tt = task % n_ttiles, ot = (task / n_ttiles) % n_otiles, h = task / (n_ttiles * n_otiles);
+  const int r16 = lane & 15, q4 = lane >> 4;
+  const int t = tt * 16 + r16;
+  const bool tok_ok = t < n_tok;
+  const bf16* xrow = in + ((size_t)(tok_ok ? t : 0) * H + h) * in_stride;
+  const bf16* wrow[4];
+  bool o_ok[4];
+#pragma unroll
+  for (int mt = 0; mt < 4; ++mt) {
+    const int o = ot * 64 + mt * 16 + r16;
+    o_ok[mt] = o < NO;
+    wrow[mt] = wo + ((size_t)h * NO + (o_ok[mt] ? o : 0)) * NI;
+  }
+  floatx4 acc[4];
+#pragma unroll
+  for (int mt = 0; mt < 4; ++mt) acc[mt] = floatx4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll 2
+  for (int k0 = 0; k0 < NI; k0 += 32) {
+    const int i = k0 + 8 * q4;
+    const bool i_ok = i < NI;
+    hw_u32x4 xb = {0u, 0u, 0u, 0u};
+    if (tok_ok && i_ok) xb = *reinterpret_cast<const hw_u32x4*>(xrow + i);
+#pragma unroll
+    for (int mt = 0; mt < 4; ++mt) {
+      hw_u32x4 wa = {0u, 0u, 0u, 0u};
+      if (o_ok[mt] && i_ok) wa = *reinterpret_cast<const hw_u32x4*>(wrow[mt] + i);
+      acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, wa), __builtin_bit_cast(bf16x8, xb),
+                                                        acc[mt], 0, 0, 0);
+    }
+  }
+  if (!tok_ok) return;
+  const float g = gate ? gate[(size_t)t * H + h] : 1.0f;
+  bf16* orow = out + ((size_t)t * H + h) * out_stride;
+#pragma unroll
+  for (int mt = 0; mt < 4; ++mt) {
+    const int o0 = ot * 64 + mt * 16 + 4 * q4;
+    if (o0 + 3 < NO && (out_stride & 3) == 0) {
+      bf16x4 v;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) v[i] = (bf16)(acc[mt][i] * g);
+      *reinterpret_cast<bf16x4*>(orow + o0) = v;
+    } else {
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        if (o0 + i < NO) orow[o0 + i] = (bf16)(acc[mt][i] * g);
+    }
+  }
+}
+
+MF_API int mf_headwise_mfma(const void* in, int in_stride, const void* wo, void* out, int out_stride,
+                            const float* gate, int n_tok, int H, int NI, int NO, hipStream_t stream) {
+  if (n_tok <= 0) return 0;
+  if (H < 1 || NI < 1 || NO < 1 || NI % 8 || in_stride % 8 || (uintptr_t)in % 16 || (uintptr_t)wo % 16 ||
+      (uintptr_t)out % 8)
+    return (int)hipErrorInvalidValue;
+  const int n_ttiles = (n_tok + 15) / 16, n_otiles = (NO + 63) / 64;
+  const long long tasks = (long long)H * n_otiles * n_ttiles;
+  headwise_mfma_kernel<<<(unsigned)((tasks + 3) / 4), 256, 0, stream>>>((const bf16*)in, in_stride, (const bf16*)wo,
+                                                                        (bf16*)out, out_stride, gate, n_tok, H, NI, NO,
+                                                                        n_ttiles, n_otiles);
   return mf_launch_status();
 }
 

@@ -39,10 +39,14 @@ constexpr int CT = RP / 32;           // 16-column tiles of a wave's column half
 constexpr int M = 64, TK = 32;        // rows of a workgroup, keys of a tile
 constexpr int KSTR = DKP + 8;         // LDS row strides in elements (16 bytes of padding)
 constexpr int VSTR = TK + 8;
+// a transposed row (one value column, TK keys) starts 16 bytes further for every 8 columns: the 64
+// lanes of a staging write hold 64 neighbouring blocks of 8 columns, and without the shift their
+// rows, a multiple of 128 bytes apart, would all fall on the same banks
+__device__ __forceinline__ int vt_at(int col) { return col * VSTR + (col >> 3) * 8; }
 constexpr int PSTR = TK + 8;
 constexpr int NB8 = (DKP / 8) * (TK / 8);          // 8 x 8 blocks of a tile
 constexpr int ROUNDS = (NB8 + 255) / 256;
-constexpr size_t LDS_BYTES = ((size_t)TK * KSTR + (size_t)RP * VSTR + (size_t)M * PSTR) * 2 + (2 * M + M + M) * 4;
+constexpr size_t LDS_BYTES = ((size_t)TK * KSTR + (size_t)RP * VSTR + (RP / 8) * 8 + (size_t)M * PSTR) * 2 + (2 * M + M + M) * 4;
 
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 
@@ -56,7 +60,7 @@ __global__ __launch_bounds__(256) void latent_mfma_kernel(
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   bf16* Kt = reinterpret_cast<bf16*>(smem);                 // [TK][KSTR]
   bf16* Vt = Kt + TK * KSTR;                                // [RP][VSTR]
-  bf16* Ps = Vt + RP * VSTR;                                // [M][PSTR]
+  bf16* Ps = Vt + RP * VSTR + (RP / 8) * 8;                 // [M][PSTR]
   float* smax = reinterpret_cast<float*>(Ps + M * PSTR);    // [2][M]
   float* ssum = smax + 2 * M;                               // [M]   sums of key half 1, at the end
   float* spare = ssum + M;                                  // [M]
@@ -119,14 +123,13 @@ __global__ __launch_bounds__(256) void latent_mfma_kernel(
     for (int rd = 0; rd < ROUNDS; ++rd) {
       const int blk = rd * 256 + (int)threadIdx.x;
       const int cc = blk % (DKP / 8), kg = blk / (DKP / 8);
+      const int jg = j0 + kg * 8;                  // the block's 8 keys lie in one page
+      const bool live = blk < NB8 && jg <= last_pos && cc * 8 < DK;
+      const bf16* src = cache + ((size_t)(live ? pt[jg / MF_PAGE] : 0) * MF_PAGE + jg % MF_PAGE) * DK + cc * 8;
 #pragma unroll
       for (int k = 0; k < 8; ++k) {
-        const int j = j0 + kg * 8 + k;
         u32x4 v = {0u, 0u, 0u, 0u};
-        if (blk < NB8 && j <= last_pos && cc * 8 < DK) {
-          const int page = pt[j / MF_PAGE];
-          v = *reinterpret_cast<const u32x4*>(cache + ((size_t)page * MF_PAGE + j % MF_PAGE) * DK + cc * 8);
-        }
+        if (live && jg + k <= last_pos) v = *reinterpret_cast<const u32x4*>(src + (size_t)k * DK);
         pre[rd][k] = v;
       }
     }
@@ -149,7 +152,7 @@ __global__ __launch_bounds__(256) void latent_mfma_kernel(
             const unsigned a = pre[rd][2 * j2][c >> 1], bb = pre[rd][2 * j2 + 1][c >> 1];
             tv[j2] = (c & 1) ? ((a >> 16) | (bb & 0xffff0000u)) : ((a & 0xffffu) | (bb << 16));
           }
-          *reinterpret_cast<u32x4*>(Vt + (size_t)(cc * 8 + c) * VSTR + kg * 8) = tv;
+          *reinterpret_cast<u32x4*>(Vt + vt_at(cc * 8 + c) + kg * 8) = tv;
         }
       }
     }
@@ -223,7 +226,7 @@ __global__ __launch_bounds__(256) void latent_mfma_kernel(
 #pragma unroll
     for (int c = 0; c < CT; ++c) {
       const int col = wk * (RP / 2) + 16 * c + r16;
-      const bf16x8 vf = as_bf16x8(*reinterpret_cast<const u32x4*>(Vt + (size_t)col * VSTR + 8 * q4));
+      const bf16x8 vf = as_bf16x8(*reinterpret_cast<const u32x4*>(Vt + vt_at(col) + 8 * q4));
       o[0][c] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pf[0], o[0][c], 0, 0, 0);
       o[1][c] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pf[1], o[1][c], 0, 0, 0);
     }

@@ -16,7 +16,7 @@
 // chunk edges fall inside the step, never on what else is in the batch.
 #include "common.h"
 
-#define MF_SCAN_CHUNK 64
+#define MF_SCAN_CHUNK 32
 
 __device__ __forceinline__ float sigmoid_f(float x) { return 1.0f / (1.0f + expf(-x)); }
 
@@ -60,6 +60,7 @@ __global__ __launch_bounds__(256) void mingru_chunk_reduce_kernel(const float* _
   if (ch >= W) return;
   const int t0 = chunk_t0[c], n = chunk_n[c];
   float A = 1.f, B = 0.f;
+#pragma unroll 4
   for (int i = 0; i < n; ++i) {
     const float* row = zug + (size_t)(t0 + i) * 3 * W + ch;
     float a, b;
@@ -86,9 +87,11 @@ __global__ __launch_bounds__(256) void mingru_chunk_apply_kernel(
   if (ch >= W) return;
   const int seq = chunk_seq[c];
   float S = state_in[(size_t)seq * W + ch];
+#pragma unroll 4
   for (int k = chunk_first[c]; k < c; ++k)
     S = ab[((size_t)k * 2) * W + ch] * S + ab[((size_t)k * 2 + 1) * W + ch];
   const int t0 = chunk_t0[c], n = chunk_n[c];
+#pragma unroll 4
   for (int i = 0; i < n; ++i) {
     const float* row = zug + (size_t)(t0 + i) * 3 * W + ch;
     float a, b;

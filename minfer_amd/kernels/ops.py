@@ -53,6 +53,7 @@ _PROTOTYPES = {
         "mf_latent_prep": [_P, c_int, c_int, c_int, _P, c_float, _P, _P, c_int, _P, _P, _P, c_int, _P, _P, _P, _P,
                            c_int, c_int, c_int, c_int, c_int, c_int, c_int, _P],
         "mf_headwise_linear": [_P, c_int, _P, _P, c_int, _P, c_int, c_int, c_int, c_int, c_int, _P],
+        "mf_headwise_mfma": [_P, c_int, _P, _P, c_int, _P, c_int, c_int, c_int, c_int, _P],
         "mf_latent_attn": [_P, _P, _P, c_int, _P, _P, _P, _P, c_int, c_int, c_int, c_int, c_int, c_float, c_int,
                            c_int, c_int, _P],
     },
@@ -495,7 +496,7 @@ def rope_pairs_inplace(qkv: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor, 
 
 
 # ------------------------------------------------------------------ recurrences
-SCAN_CHUNK = 64          # tokens of a chunk of the chunked scan (MF_SCAN_CHUNK in csrc/recurrence.hip)
+SCAN_CHUNK = 32          # tokens of a chunk of the chunked scan (MF_SCAN_CHUNK in csrc/recurrence.hip)
 
 
 def scan_chunks(host_new):
@@ -604,6 +605,31 @@ def headwise_linear(x: torch.Tensor, n_in: int, wt: torch.Tensor, out: torch.Ten
     _check(_fn("attn_latent", "mf_headwise_linear")(_ptr(x), in_stride, _ptr(wt), _ptr(out), out.shape[2], _ptr(gate),
                                                      _is_bf16(x), n_tok, heads, n_in, n_out, _stream()),
            "headwise_linear")
+
+
+def headwise_mfma_takes(dtype, n_in: int, in_stride: int) -> bool:
+    """Whether `headwise_linear_mfma` runs these sizes: bfloat16 and inputs in 16-byte pieces."""
+    return dtype == torch.bfloat16 and n_in % 8 == 0 and in_stride % 8 == 0
+
+
+def headwise_linear_mfma(x: torch.Tensor, n_in: int, wo: torch.Tensor, out: torch.Tensor, n_out: int,
+                         gate: Optional[torch.Tensor] = None) -> None:
+    """`headwise_linear` on the matrix cores: `wo` is `[heads][n_out][n_in]` (each head's matrix
+    output-major), everything bfloat16, n_in and x's row length multiples of 8."""
+    _need(x, "headwise_linear_mfma.x", torch.bfloat16)
+    if x.dim() != 3 or out.dim() != 3:
+        raise KernelError("headwise_linear_mfma: x and out are [tokens][heads][row]")
+    n_tok, heads, in_stride = x.shape
+    _need(wo, "headwise_linear_mfma.wo", torch.bfloat16, (heads, n_out, n_in))
+    _need(out, "headwise_linear_mfma.out", torch.bfloat16)
+    if tuple(out.shape[:2]) != (n_tok, heads) or out.shape[2] < n_out or in_stride < n_in:
+        raise KernelError(f"headwise_linear_mfma: x {tuple(x.shape)}, out {tuple(out.shape)}, matrix {tuple(wo.shape)}")
+    if not headwise_mfma_takes(x.dtype, n_in, in_stride):
+        raise KernelError(f"headwise_linear_mfma: inputs of {n_in} in rows of {in_stride} are not 16-byte pieces")
+    if gate is not None:
+        _need(gate, "headwise_linear_mfma.gate", torch.float32, (n_tok, heads))
+    _check(_fn("attn_latent", "mf_headwise_mfma")(_ptr(x), in_stride, _ptr(wo), _ptr(out), out.shape[2], _ptr(gate),
+                                                   n_tok, heads, n_in, n_out, _stream()), "headwise_linear_mfma")
 
 
 def latent_split_plan(n_blocks: int, max_len: int, target_blocks: Optional[int] = None) -> Tuple[int, int]:

@@ -64,10 +64,14 @@ class LatentAttention(Mixer):
         self.off_dkv = H * (self.dn + self.dr)
         self.off_gate = self.off_dkv + self.dk
         self.latent_weight = get(n["dkv_norm"]).to(torch.float32).contiguous()
-        # per-head matrices, input-major: uk_t[h] = Wuk_h [dim][rank] takes q_plain to the latent's
-        # side; uv_t[h] = Wuv_h^T [rank][v_dim] takes the result over the latents to the head's values
-        self.uk_t = get(n["uk"]).view(H, self.dn, self.rank).contiguous()
-        self.uv_t = get(n["uv"]).view(H, self.dv, self.rank).transpose(1, 2).contiguous()
+        # per-head matrices: Wuk_h^T takes q_plain to the latent's side, Wuv_h takes the result over
+        # the latents to the head's values.  The matrix-core kernel reads them output-major
+        # ([rank][dim], [v_dim][rank]), the plain one input-major.
+        uk, uv = get(n["uk"]).view(H, self.dn, self.rank), get(n["uv"]).view(H, self.dv, self.rank)
+        self.uk_mfma = ops.headwise_mfma_takes(uk.dtype, self.dn, self.dn) and self.rt.is_bf16
+        self.uv_mfma = ops.headwise_mfma_takes(uv.dtype, self.rank, self.rank) and self.rt.is_bf16
+        self.uk_t = (uk.transpose(1, 2) if self.uk_mfma else uk).contiguous()
+        self.uv_t = (uv if self.uv_mfma else uv.transpose(1, 2)).contiguous()
         self.o = Linear(get(n["o"]))
 
     def cache_request(self):
@@ -91,10 +95,11 @@ class LatentAttention(Mixer):
         gate = torch.empty((n, H), dtype=torch.float32, device=dev)
         ops.latent_prep(proj, self.off_dkv, self.off_gate, self.latent_weight, self.eps, cos, sin, ctx.positions,
                         ctx.seq_of_tok, table, rows, q_plain, q_abs, gate, H, self.dn, self.dr, self.rank, writes_cache)
-        ops.headwise_linear(q_plain, self.dn, self.uk_t, q_abs, self.rank)
+        (ops.headwise_linear_mfma if self.uk_mfma else ops.headwise_linear)(q_plain, self.dn, self.uk_t, q_abs, self.rank)
         o_lat = torch.empty((n, H, self.rank), dtype=dt, device=dev)
         ops.latent_attn(q_abs, rows, table, ctx.positions, ctx.seq_of_tok, o_lat, self.rank, self.scale,
                         0 if self.window is None else int(self.window), ctx.max_len, ctx=ctx)
         o = torch.empty((n, H, self.dv), dtype=dt, device=dev)
-        ops.headwise_linear(o_lat, self.rank, self.uv_t, o, self.dv, gate=gate)
+        (ops.headwise_linear_mfma if self.uv_mfma else ops.headwise_linear)(o_lat, self.rank, self.uv_t, o, self.dv,
+                                                                             gate=gate)
         self.o(o.view(n, H * self.dv), out=h, accumulate=accumulate)

@@ -296,6 +296,14 @@ def headwise_linear(x, n_in, wt, out, n_out, gate=None):
     out[:, :, :n_out] = y.to(out.dtype)
 
 
+def headwise_mfma_takes(dtype, n_in, in_stride):
+    return dtype == torch.bfloat16 and n_in % 8 == 0 and in_stride % 8 == 0
+
+
+def headwise_linear_mfma(x, n_in, wo, out, n_out, gate=None):
+    headwise_linear(x, n_in, wo.transpose(1, 2), out, n_out, gate)
+
+
 def latent_attn(q_abs, cache, page_table, positions, seq_of_tok, out, rank, scale, window, max_len, ctx=None):
     t, heads, dk = q_abs.shape
     flat = cache.view(-1, PAGE, dk)
@@ -381,7 +389,7 @@ NAMES = ["embed", "rmsnorm", "gather_rows", "swiglu", "convert", "fill_normal", 
          "rope_kvwrite", "rope_inplace", "linear", "attn_tokens", "attn_prefill", "argmax", "sample", "penalties",
          "top_k", "top_p", "sample_filtered", "sample_filtered_takes", "advance", "interleave_gate_up", "linear_swiglu", "linear_normed", "linear_fused", "attn_decode_rope",
          "group_rmsnorm", "xielu", "rope_table_freqs", "rope_pairs_inplace", "mingru_scan", "latent_prep",
-         "headwise_linear", "latent_attn"]
+         "headwise_linear", "latent_attn", "headwise_mfma_takes", "headwise_linear_mfma"]
 
 
 def install(monkeypatch):

@@ -147,6 +147,22 @@ def test_headwise_linear_kernel():
         assert got[:, :, 290:].abs().max() == 0
 
 
+@pytest.mark.parametrize("n_tok, heads, n_in, n_out, stride", [(11, 3, 40, 290, 48), (1, 16, 128, 512, 128),
+                                                              (100, 5, 72, 8, 72), (8, 2, 264, 40, 264)])
+def test_headwise_linear_matrix_core_kernel(n_tok, heads, n_in, n_out, stride):
+    from minfer_amd.kernels import ops
+    x = rnd(n_tok, heads, stride, seed=8).to(torch.bfloat16)
+    wo = rnd(heads, n_out, n_in, seed=9, scale=0.2).to(torch.bfloat16)
+    gate = torch.rand(n_tok, heads, generator=torch.Generator().manual_seed(1))
+    for g in (None, gate):
+        want = torch.zeros(n_tok, heads, n_out + 4, dtype=torch.bfloat16)
+        plain_ops.headwise_linear_mfma(x, n_in, wo, want, n_out, g)
+        got = torch.zeros(n_tok, heads, n_out + 4, dtype=torch.bfloat16, device=DEV)
+        ops.headwise_linear_mfma(x.to(DEV), n_in, wo.to(DEV), got, n_out, None if g is None else g.to(DEV))
+        assert ((got.cpu().float() - want.float()).abs() / (1 + want.float().abs())).max() < 1e-2
+        assert got[:, :, n_out:].abs().max() == 0
+
+
 def _latent_case(dtype, heads, rank, rot, lens, seed, needle=None):
     """Cached rows for sequences of `lens` tokens in shuffled pages of a NaN-poisoned pool, queries
     for the last few positions of each.  `needle` = (sequence, position): that row is made to
