@@ -157,13 +157,15 @@ MF_API int mf_headwise_linear(const void* in, int in_stride, const void* wt, voi
 }
 
 // The same on the matrix cores (bfloat16, NI a multiple of 8): `wo` holds each head's matrix
-// output-major ([NO][NI]).  A wave takes 16 tokens x 64 outputs of one head and forms
+// output-major ([NO][NI]).  A wave takes 16 tokens x 16 MT outputs of one head (MT = 4; 1 where a
+// step has at most 16 tokens, so that there are waves enough to have the matrices' bytes in flight) and forms
 // D^T = W X^T with 16x16x32 MFMA, operands straight from memory (a lane's 8 consecutive inputs are
 // 16 bytes of a row in both), so that a lane ends up with four neighbouring outputs of one token.
 // Tasks are numbered head, output tile, token tile (fastest): the four waves of a block share a
 // head's rows of W where the step has tokens enough, and spread over the outputs where not.
 typedef unsigned int hw_u32x4 __attribute__((ext_vector_type(4)));
 
+template <int MT>
 __global__ __launch_bounds__(256) void headwise_mfma_kernel(const bf16* __restrict__ in, int in_stride,
                                                             const bf16* __restrict__ wo, bf16* __restrict__ out,
                                                             int out_stride, const float* __restrict__ gate, int n_tok,
@@ -176,25 +178,25 @@ __global__ __launch_bounds__(256) void headwise_mfma_kernel(const bf16* __restri
   const int t = tt * 16 + r16;
   const bool tok_ok = t < n_tok;
   const bf16* xrow = in + ((size_t)(tok_ok ? t : 0) * H + h) * in_stride;
-  const bf16* wrow[4];
-  bool o_ok[4];
+  const bf16* wrow[MT];
+  bool o_ok[MT];
 #pragma unroll
-  for (int mt = 0; mt < 4; ++mt) {
-    const int o = ot * 64 + mt * 16 + r16;
+  for (int mt = 0; mt < MT; ++mt) {
+    const int o = ot * (16 * MT) + mt * 16 + r16;
     o_ok[mt] = o < NO;
     wrow[mt] = wo + ((size_t)h * NO + (o_ok[mt] ? o : 0)) * NI;
   }
-  floatx4 acc[4];
+  floatx4 acc[MT];
 #pragma unroll
-  for (int mt = 0; mt < 4; ++mt) acc[mt] = floatx4{0.f, 0.f, 0.f, 0.f};
-#pragma unroll 2
+  for (int mt = 0; mt < MT; ++mt) acc[mt] = floatx4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll 4
   for (int k0 = 0; k0 < NI; k0 += 32) {
     const int i = k0 + 8 * q4;
     const bool i_ok = i < NI;
     hw_u32x4 xb = {0u, 0u, 0u, 0u};
     if (tok_ok && i_ok) xb = *reinterpret_cast<const hw_u32x4*>(xrow + i);
 #pragma unroll
-    for (int mt = 0; mt < 4; ++mt) {
+    for (int mt = 0; mt < MT; ++mt) {
       hw_u32x4 wa = {0u, 0u, 0u, 0u};
       if (o_ok[mt] && i_ok) wa = *reinterpret_cast<const hw_u32x4*>(wrow[mt] + i);
       acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, wa), __builtin_bit_cast(bf16x8, xb),
@@ -205,8 +207,8 @@ __global__ __launch_bounds__(256) void headwise_mfma_kernel(const bf16* __restri
   const float g = gate ? gate[(size_t)t * H + h] : 1.0f;
   bf16* orow = out + ((size_t)t * H + h) * out_stride;
 #pragma unroll
-  for (int mt = 0; mt < 4; ++mt) {
-    const int o0 = ot * 64 + mt * 16 + 4 * q4;
+  for (int mt = 0; mt < MT; ++mt) {
+    const int o0 = ot * (16 * MT) + mt * 16 + 4 * q4;
     if (o0 + 3 < NO && (out_stride & 3) == 0) {
       bf16x4 v;
 #pragma unroll
@@ -226,11 +228,18 @@ MF_API int mf_headwise_mfma(const void* in, int in_stride, const void* wo, void*
   if (H < 1 || NI < 1 || NO < 1 || NI % 8 || in_stride % 8 || (uintptr_t)in % 16 || (uintptr_t)wo % 16 ||
       (uintptr_t)out % 8)
     return (int)hipErrorInvalidValue;
-  const int n_ttiles = (n_tok + 15) / 16, n_otiles = (NO + 63) / 64;
-  const long long tasks = (long long)H * n_otiles * n_ttiles;
-  headwise_mfma_kernel<<<(unsigned)((tasks + 3) / 4), 256, 0, stream>>>((const bf16*)in, in_stride, (const bf16*)wo,
-                                                                        (bf16*)out, out_stride, gate, n_tok, H, NI, NO,
-                                                                        n_ttiles, n_otiles);
+  const int n_ttiles = (n_tok + 15) / 16;
+  if (n_tok <= 16) {
+    const int n_otiles = (NO + 15) / 16;
+    const long long tasks = (long long)H * n_otiles * n_ttiles;
+    headwise_mfma_kernel<1><<<(unsigned)((tasks + 3) / 4), 256, 0, stream>>>(
+        (const bf16*)in, in_stride, (const bf16*)wo, (bf16*)out, out_stride, gate, n_tok, H, NI, NO, n_ttiles, n_otiles);
+  } else {
+    const int n_otiles = (NO + 63) / 64;
+    const long long tasks = (long long)H * n_otiles * n_ttiles;
+    headwise_mfma_kernel<4><<<(unsigned)((tasks + 3) / 4), 256, 0, stream>>>(
+        (const bf16*)in, in_stride, (const bf16*)wo, (bf16*)out, out_stride, gate, n_tok, H, NI, NO, n_ttiles, n_otiles);
+  }
   return mf_launch_status();
 }
 

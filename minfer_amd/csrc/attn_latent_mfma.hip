@@ -10,14 +10,15 @@
 // up to multiples of 32), so queries and accumulators live in registers; the host asks for the
 // variant a model needs the first time it runs.
 //
-// A workgroup of 4 waves walks the keys in tiles of 32.  A tile is loaded into registers a tile
-// ahead, then written to LDS twice: as it is ([key][d], for q . k) and transposed ([column][key],
-// for p . v: the matrix cores want the contracted index contiguous in both operands; the
-// transposition is 8 x 8 blocks turned in registers).  Wave (wr, wk) forms the scores of row half
-// wr against key half wk as S^T = K Q^T, so that a lane ends up with four keys of one row; the
-// two key halves exchange their row maxima through LDS; the probabilities go to LDS in bfloat16;
-// wave (wr, wc) then adds P V for row half wr and column half wc as O^T = V^T P^T, where a lane
-// again owns one row, so the running maximum, the rescaling and the sum stay in the lane.
+// A workgroup of 4 waves walks the keys in tiles of 32; wave w owns rows 16 w .. 16 w + 15.  A tile
+// is loaded into registers a tile ahead, then written to LDS twice: as it is ([key][d], for
+// q . k) and transposed ([column][key], for p . v: the matrix cores want the contracted index
+// contiguous in both operands; the transposition is 8 x 8 blocks turned in registers).  A wave
+// forms its rows' scores against the tile as S^T = K Q^T (two products of 16 keys), so that lane
+// (r, q) ends up with keys 4 q .. 4 q + 3 and 16 + 4 q .. 16 + 4 q + 3 of row r: the softmax of a
+// row stays inside its wave, and the eight probabilities of a lane are, as they lie, its share of
+// the second product's operand, O^T = V^T P^T, with the keys taken in that same order from the
+// transposed tile.  Nothing but the tile passes through LDS, and a tile costs two barriers.
 // 16x16x32 MFMA throughout; scores, statistics and accumulators 32-bit.
 //
 // Keys behind a sequence's last position (the rest of its last page) are written to LDS as zeros:
@@ -35,7 +36,7 @@ namespace latm {
 
 constexpr int DKP = MF_LAT_DKP, RP = MF_LAT_RP;
 constexpr int KS = DKP / 32;          // k steps of a score product
-constexpr int CT = RP / 32;           // 16-column tiles of a wave's column half
+constexpr int CT = RP / 16;           // 16-column tiles of the values
 constexpr int M = 64, TK = 32;        // rows of a workgroup, keys of a tile
 constexpr int KSTR = DKP + 8;         // LDS row strides in elements (16 bytes of padding)
 constexpr int VSTR = TK + 8;
@@ -43,10 +44,9 @@ constexpr int VSTR = TK + 8;
 // lanes of a staging write hold 64 neighbouring blocks of 8 columns, and without the shift their
 // rows, a multiple of 128 bytes apart, would all fall on the same banks
 __device__ __forceinline__ int vt_at(int col) { return col * VSTR + (col >> 3) * 8; }
-constexpr int PSTR = TK + 8;
 constexpr int NB8 = (DKP / 8) * (TK / 8);          // 8 x 8 blocks of a tile
 constexpr int ROUNDS = (NB8 + 255) / 256;
-constexpr size_t LDS_BYTES = ((size_t)TK * KSTR + (size_t)RP * VSTR + (RP / 8) * 8 + (size_t)M * PSTR) * 2 + (2 * M + M + M) * 4;
+constexpr size_t LDS_BYTES = ((size_t)TK * KSTR + (size_t)RP * VSTR + (RP / 8) * 8) * 2;
 
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 
@@ -60,14 +60,9 @@ __global__ __launch_bounds__(256) void latent_mfma_kernel(
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   bf16* Kt = reinterpret_cast<bf16*>(smem);                 // [TK][KSTR]
   bf16* Vt = Kt + TK * KSTR;                                // [RP][VSTR]
-  bf16* Ps = Vt + RP * VSTR + (RP / 8) * 8;                 // [M][PSTR]
-  float* smax = reinterpret_cast<float*>(Ps + M * PSTR);    // [2][M]
-  float* ssum = smax + 2 * M;                               // [M]   sums of key half 1, at the end
-  float* spare = ssum + M;                                  // [M]
 
   const int lane = threadIdx.x & 63;
   const int w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  const int wr = w >> 1, wk = w & 1;
   const int r16 = lane & 15, q4 = lane >> 4;
 
   const int b = tile_seq ? tile_seq[blockIdx.x] : (int)blockIdx.x;
@@ -84,36 +79,29 @@ __global__ __launch_bounds__(256) void latent_mfma_kernel(
   const int j_begin = max(lo_all, split * split_len);
   const int j_end = min(last_pos + 1, (split + 1) * split_len);
 
-  // this lane's two rows (one per row tile), their positions and queries
-  int row_pos[2], row_lo[2];
-  size_t row_th[2];
-  bool row_ok[2];
-  bf16x8 qf[2][KS];
-#pragma unroll
-  for (int rt = 0; rt < 2; ++rt) {
-    const int r = 32 * wr + 16 * rt + r16;
-    const int tq = r / HC, hh = r % HC;
-    row_ok[rt] = tq < n_here && hh < hcount;
-    const int t = t_first + (row_ok[rt] ? tq : 0);
-    row_pos[rt] = row_ok[rt] ? first_pos + tq : -1;
-    row_lo[rt] = window > 0 ? max(0, row_pos[rt] - window + 1) : 0;
-    row_th[rt] = (size_t)t * H + h0 + (row_ok[rt] ? hh : 0);
-    const bf16* qrow = q_abs + row_th[rt] * DK;
+  // this lane's row, its position and query
+  const int r = 16 * w + r16;
+  const int tq = r / HC, hh = r % HC;
+  const bool row_ok = tq < n_here && hh < hcount;
+  const int row_pos = row_ok ? first_pos + tq : -1;
+  const int row_lo = window > 0 ? max(0, row_pos - window + 1) : 0;
+  const size_t row_th = (size_t)(t_first + (row_ok ? tq : 0)) * H + h0 + (row_ok ? hh : 0);
+  const bool wave_live = 16 * w < n_here * HC;        // some row of this wave exists
+  bf16x8 qf[KS];
+  {
+    const bf16* qrow = q_abs + row_th * DK;
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
       const int d = 32 * ks + 8 * q4;
       u32x4 v = {0u, 0u, 0u, 0u};
-      if (row_ok[rt] && d < DK) v = *reinterpret_cast<const u32x4*>(qrow + d);
-      qf[rt][ks] = as_bf16x8(v);
+      if (row_ok && d < DK) v = *reinterpret_cast<const u32x4*>(qrow + d);
+      qf[ks] = as_bf16x8(v);
     }
   }
-
-  floatx4 o[2][CT];
+  floatx4 o[CT];
 #pragma unroll
-  for (int rt = 0; rt < 2; ++rt)
-#pragma unroll
-    for (int c = 0; c < CT; ++c) o[rt][c] = floatx4{0.f, 0.f, 0.f, 0.f};
-  float m_run[2] = {-INFINITY, -INFINITY}, l_run[2] = {0.f, 0.f};
+  for (int c = 0; c < CT; ++c) o[c] = floatx4{0.f, 0.f, 0.f, 0.f};
+  float m_run = -INFINITY, l_run = 0.f;
 
   // a tile ahead, in registers: 8 x 8 blocks (8 keys x 8 columns), block `blk` of a round is
   // column chunk blk % (DKP/8) of key group blk / (DKP/8)
@@ -166,130 +154,115 @@ __global__ __launch_bounds__(256) void latent_mfma_kernel(
     if (j0 + TK < j_end) fetch(j0 + TK);
     __syncthreads();
 
-    // scores: S^T (keys x rows) for key half wk, row half wr
-    floatx4 s[2] = {floatx4{0.f, 0.f, 0.f, 0.f}, floatx4{0.f, 0.f, 0.f, 0.f}};
+    if (!wave_live) continue;            // (uniform over the wave; the barriers above are passed by all)
+    // scores: S^T (keys x rows), keys 0..15 and 16..31 of the tile
+    floatx4 s2[2] = {floatx4{0.f, 0.f, 0.f, 0.f}, floatx4{0.f, 0.f, 0.f, 0.f}};
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
-      const bf16x8 kf = as_bf16x8(*reinterpret_cast<const u32x4*>(Kt + (size_t)(16 * wk + r16) * KSTR + 32 * ks + 8 * q4));
-      s[0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qf[0][ks], s[0], 0, 0, 0);
-      s[1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qf[1][ks], s[1], 0, 0, 0);
+      const bf16x8 k0f = as_bf16x8(*reinterpret_cast<const u32x4*>(Kt + (size_t)r16 * KSTR + 32 * ks + 8 * q4));
+      const bf16x8 k1f = as_bf16x8(*reinterpret_cast<const u32x4*>(Kt + (size_t)(16 + r16) * KSTR + 32 * ks + 8 * q4));
+      s2[0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(k0f, qf[ks], s2[0], 0, 0, 0);
+      s2[1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(k1f, qf[ks], s2[1], 0, 0, 0);
     }
-    // lane (r16, q4): row 32 wr + 16 rt + r16, keys j0 + 16 wk + 4 q4 + i
-    float mloc[2];
+    // lane (r16, q4): row 16 w + r16, keys j0 + 16 kt + 4 q4 + i
+    float mx = -INFINITY;
 #pragma unroll
-    for (int rt = 0; rt < 2; ++rt) {
-      float mx = -INFINITY;
+    for (int kt = 0; kt < 2; ++kt)
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        const int j = j0 + 16 * wk + 4 * q4 + i;
-        const bool ok = row_ok[rt] && j >= j_begin && j < j_end && j <= row_pos[rt] && j >= row_lo[rt];
-        s[rt][i] = ok ? s[rt][i] * scale : -INFINITY;
-        mx = fmaxf(mx, s[rt][i]);
+        const int j = j0 + 16 * kt + 4 * q4 + i;
+        const bool ok = row_ok && j >= j_begin && j < j_end && j <= row_pos && j >= row_lo;
+        s2[kt][i] = ok ? s2[kt][i] * scale : -INFINITY;
+        mx = fmaxf(mx, s2[kt][i]);
       }
-      mx = fmaxf(mx, __shfl_xor(mx, 16, MF_WAVE));
-      mx = fmaxf(mx, __shfl_xor(mx, 32, MF_WAVE));
-      mloc[rt] = mx;
-      if (q4 == 0) smax[wk * M + 32 * wr + 16 * rt + r16] = mx;
-    }
-    __syncthreads();
-    float corr[2];
+    mx = fmaxf(mx, __shfl_xor(mx, 16, MF_WAVE));
+    mx = fmaxf(mx, __shfl_xor(mx, 32, MF_WAVE));
+    const float m_new = fmaxf(m_run, mx);
+    const float corr = (m_new == -INFINITY) ? 1.f : __expf(m_run - m_new);
+    float ps = 0.f;
+    bf16x8 pf;
 #pragma unroll
-    for (int rt = 0; rt < 2; ++rt) {
-      const int r = 32 * wr + 16 * rt + r16;
-      const float m_new = fmaxf(m_run[rt], fmaxf(mloc[rt], smax[(wk ^ 1) * M + r]));
-      corr[rt] = (m_new == -INFINITY) ? 1.f : __expf(m_run[rt] - m_new);
-      float ps = 0.f;
-      bf16x4 pv;
+    for (int kt = 0; kt < 2; ++kt)
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        const float pe = (s[rt][i] == -INFINITY) ? 0.f : __expf(s[rt][i] - m_new);
+        const float pe = (s2[kt][i] == -INFINITY) ? 0.f : __expf(s2[kt][i] - m_new);
         ps += pe;
-        pv[i] = (bf16)pe;
+        pf[4 * kt + i] = (bf16)pe;
       }
-      ps += __shfl_xor(ps, 16, MF_WAVE);
-      ps += __shfl_xor(ps, 32, MF_WAVE);
-      l_run[rt] = l_run[rt] * corr[rt] + ps;       // of this wave's key half only; the halves meet at the end
-      m_run[rt] = m_new;
-      *reinterpret_cast<bf16x4*>(Ps + (size_t)r * PSTR + 16 * wk + 4 * q4) = pv;
-    }
-    __syncthreads();
-
-    // O^T (columns x rows) += V^T P^T for row half wr, column half wc = wk
-#pragma unroll
-    for (int rt = 0; rt < 2; ++rt)
-#pragma unroll
-      for (int c = 0; c < CT; ++c) o[rt][c] *= corr[rt];
-    bf16x8 pf[2];
-#pragma unroll
-    for (int rt = 0; rt < 2; ++rt)
-      pf[rt] = as_bf16x8(*reinterpret_cast<const u32x4*>(Ps + (size_t)(32 * wr + 16 * rt + r16) * PSTR + 8 * q4));
+    ps += __shfl_xor(ps, 16, MF_WAVE);
+    ps += __shfl_xor(ps, 32, MF_WAVE);
+    l_run = l_run * corr + ps;
+    m_run = m_new;
+    // O^T (columns x rows) += V^T P^T; the lane's eight keys are 4 q4 .. + 3 and 16 + 4 q4 .. + 3
 #pragma unroll
     for (int c = 0; c < CT; ++c) {
-      const int col = wk * (RP / 2) + 16 * c + r16;
-      const bf16x8 vf = as_bf16x8(*reinterpret_cast<const u32x4*>(Vt + vt_at(col) + 8 * q4));
-      o[0][c] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pf[0], o[0][c], 0, 0, 0);
-      o[1][c] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pf[1], o[1][c], 0, 0, 0);
+      o[c] *= corr;
+      const bf16* vrow = Vt + vt_at(16 * c + r16) + 4 * q4;
+      typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
+      const u32x2 lo2 = *reinterpret_cast<const u32x2*>(vrow), hi2 = *reinterpret_cast<const u32x2*>(vrow + 16);
+      const u32x4 both = {lo2[0], lo2[1], hi2[0], hi2[1]};
+      o[c] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(both), pf, o[c], 0, 0, 0);
     }
   }
 
-  // the two key halves' sums meet: wave (wr, 1) hands its sums to (wr, 0) and back
-  __syncthreads();
+  // lane (r16, q4): row 16 w + r16, columns 16 c + 4 q4 + i
+  if (!row_ok) return;
+  if (n_splits == 1) {
+    const float inv = l_run > 0.f ? 1.0f / l_run : 0.f;
+    bf16* orow = out + row_th * R;
 #pragma unroll
-  for (int rt = 0; rt < 2; ++rt)
-    if (q4 == 0) (wk ? ssum : spare)[32 * wr + 16 * rt + r16] = l_run[rt];
-  __syncthreads();
-  // lane (r16, q4) of wave (wr, wc = wk): row 32 wr + 16 rt + r16, columns wc RP/2 + 16 c + 4 q4 + i
+    for (int c = 0; c < CT; ++c) {
+      const int col = 16 * c + 4 * q4;
+      if (col < R) {                        // R is a multiple of 8: the four columns go together
+        bf16x4 v;
 #pragma unroll
-  for (int rt = 0; rt < 2; ++rt) {
-    if (!row_ok[rt]) continue;
-    const int r = 32 * wr + 16 * rt + r16;
-    const float L = ssum[r] + spare[r];
-    if (n_splits == 1) {
-      const float inv = L > 0.f ? 1.0f / L : 0.f;
-      bf16* orow = out + row_th[rt] * R;
-#pragma unroll
-      for (int c = 0; c < CT; ++c) {
-        const int col = wk * (RP / 2) + 16 * c + 4 * q4;
-        if (col < R) {                      // R is a multiple of 8: the four columns go together
-          bf16x4 v;
-#pragma unroll
-          for (int i = 0; i < 4; ++i) v[i] = (bf16)(o[rt][c][i] * inv);
-          *reinterpret_cast<bf16x4*>(orow + col) = v;
-        }
+        for (int i = 0; i < 4; ++i) v[i] = (bf16)(o[c][i] * inv);
+        *reinterpret_cast<bf16x4*>(orow + col) = v;
       }
-    } else {
-      float* prow = part + (row_th[rt] * n_splits + split) * (size_t)(R + 2);
-#pragma unroll
-      for (int c = 0; c < CT; ++c) {
-        const int col = wk * (RP / 2) + 16 * c + 4 * q4;
-        if (col < R) {
-#pragma unroll
-          for (int i = 0; i < 4; ++i) prow[col + i] = o[rt][c][i];
-        }
-      }
-      if (wk == 0 && q4 == 0) { prow[R] = m_run[rt]; prow[R + 1] = L; }
     }
+  } else {
+    float* prow = part + (row_th * n_splits + split) * (size_t)(R + 2);
+#pragma unroll
+    for (int c = 0; c < CT; ++c) {
+      const int col = 16 * c + 4 * q4;
+      if (col < R) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) prow[col + i] = o[c][i];
+      }
+    }
+    if (q4 == 0) { prow[R] = m_run; prow[R + 1] = l_run; }
   }
 }
 
-// out[th][e] = sum_s acc_s[e] exp(m_s - M) / sum_s l_s exp(m_s - M), the splits in their order
+// out[th][e] = sum_s acc_s[e] exp(m_s - M) / sum_s l_s exp(m_s - M), the splits in their order (at
+// most 64).  Lane s weighs split s (every wave for itself); a thread then adds its columns' weighted
+// sums over the splits that had keys, eight loads in flight.
 __global__ __launch_bounds__(256) void latent_mfma_combine_kernel(const float* __restrict__ part,
                                                                   bf16* __restrict__ out, int R, int n_splits) {
   const size_t th = blockIdx.x;
   const float* base = part + th * n_splits * (size_t)(R + 2);
-  float Mx = -INFINITY;
-  for (int s = 0; s < n_splits; ++s) Mx = fmaxf(Mx, base[(size_t)s * (R + 2) + R]);
+  const int lane = threadIdx.x & 63;
+  const float ms = lane < n_splits ? base[(size_t)lane * (R + 2) + R] : -INFINITY;
+  const float ls = lane < n_splits ? base[(size_t)lane * (R + 2) + R + 1] : 0.f;
+  const float Mx = wave_max(ms);
+  const float wv = (ms == -INFINITY) ? 0.f : __expf(ms - Mx);
+  const unsigned long long with_keys = __ballot(ms != -INFINITY);
+  const int n_used = with_keys ? 64 - __clzll((long long)with_keys) : 0;
+  auto of_split = [](float x, int s) { return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(x), s)); };
   float L = 0.f;
-  for (int s = 0; s < n_splits; ++s) {
-    const float ms = base[(size_t)s * (R + 2) + R];
-    if (ms != -INFINITY) L += base[(size_t)s * (R + 2) + R + 1] * __expf(ms - Mx);
-  }
+  for (int s = 0; s < n_used; ++s) L += of_split(ls, s) * of_split(wv, s);
   const float inv = L > 0.f ? 1.0f / L : 0.f;
   for (int e = threadIdx.x; e < R; e += 256) {
     float a = 0.f;
-    for (int s = 0; s < n_splits; ++s) {
-      const float ms = base[(size_t)s * (R + 2) + R];
-      if (ms != -INFINITY) a += base[(size_t)s * (R + 2) + e] * __expf(ms - Mx);
+    for (int s0 = 0; s0 < n_used; s0 += 8) {
+      float wgt[8], v[8];
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        wgt[j] = s0 + j < 64 ? of_split(wv, (s0 + j) & 63) : 0.f;
+        v[j] = base[(wgt[j] != 0.f ? (size_t)(s0 + j) * (R + 2) : 0) + e];
+      }
+#pragma unroll
+      for (int j = 0; j < 8; ++j) a += (wgt[j] != 0.f ? v[j] : 0.f) * wgt[j];
     }
     out[th * R + e] = (bf16)(a * inv);
   }
@@ -312,7 +285,7 @@ MF_API int mf_latent_mfma(const void* q_abs, const void* cache, const int* page_
   using namespace latm;
   if (n_tiles <= 0) return 0;
   if (DK > DKP || DK + 31 < DKP || R > RP || R + 31 < RP || R % 8 || DK % 8 || R > DK || HC < 1 || TQ < 1 ||
-      HC * TQ > M || n_splits < 1 || split_len < TK || split_len % TK || (n_splits > 1 && !part) ||
+      HC * TQ > M || n_splits < 1 || n_splits > 64 || split_len < TK || split_len % TK || (n_splits > 1 && !part) ||
       (uintptr_t)q_abs % 16 || (uintptr_t)cache % 16 || (uintptr_t)out % 8)
     return (int)hipErrorInvalidValue;
   static bool raised = false;

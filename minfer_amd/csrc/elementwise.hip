@@ -123,6 +123,37 @@ __global__ __launch_bounds__(256) void group_rmsnorm_kernel(const float* x,
   OT* o = out + (size_t)row * d;
   bf16* co = cast_out ? cast_out + (size_t)row * d : nullptr;
   const int part = d / groups;
+  // a number of groups that is a power of two up to 256: every group has 256 / groups threads of its
+  // own and all groups go at once (a row's loads are all in flight together); else group by group
+  if ((groups & (groups - 1)) == 0 && groups <= 256) {
+    const int tpg = 256 / groups;                  // threads of a group: a power of two
+    const int g = threadIdx.x / tpg, tl = threadIdx.x % tpg;
+    const int lo = g * part;
+    float ss = 0.f;
+    for (int i = tl; i < part; i += tpg) {
+      const float v = xr[lo + i];
+      ss = fmaf(v, v, ss);
+    }
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1)
+      if (off < tpg) ss += __shfl_xor(ss, off, MF_WAVE);
+    if (tpg > 64) {                                // the group's waves meet in LDS
+      const int wv = threadIdx.x >> 6;
+      if ((threadIdx.x & 63) == 0) scratch[wv] = ss;
+      __syncthreads();
+      const int w0 = (wv / (tpg / 64)) * (tpg / 64);
+      ss = 0.f;
+      for (int k = 0; k < tpg / 64; ++k) ss += scratch[w0 + k];
+    }
+    const float scale = 1.0f / sqrtf(ss / (float)part + eps);
+    for (int i = tl; i < part; i += tpg) {
+      float y = xr[lo + i] * scale * (w ? w[lo + i] : 1.0f);
+      if (ADD) y += to_f32(o[lo + i]);
+      o[lo + i] = from_f32<OT>(y);
+      if (co) co[lo + i] = (bf16)y;
+    }
+    return;
+  }
   for (int g = 0; g < groups; ++g) {
     const int lo = g * part;
     float ss = 0.f;

@@ -632,12 +632,12 @@ def headwise_linear_mfma(x: torch.Tensor, n_in: int, wo: torch.Tensor, out: torc
                                                    n_tok, heads, n_in, n_out, _stream()), "headwise_linear_mfma")
 
 
-def latent_split_plan(n_blocks: int, max_len: int, target_blocks: Optional[int] = None) -> Tuple[int, int]:
+def latent_split_plan(n_blocks: int, max_len: int, target_blocks: Optional[int] = None, most: int = 64) -> Tuple[int, int]:
     """(n_splits, split_len) of the latent attention's keys: as many splits (whole pages, at most
-    64) as it takes to give every CU a block where the step's `n_blocks` alone do not."""
-    target = target_blocks or 2 * cu_count()
+    `most`) as it takes to give every CU a block where the step's `n_blocks` alone do not."""
+    target = target_blocks or cu_count()
     pages = (max_len + PAGE - 1) // PAGE
-    want = max(1, min(64, pages, target // max(1, n_blocks)))
+    want = max(1, min(most, pages, target // max(1, n_blocks)))
     per = (pages + want - 1) // want
     return (pages + per - 1) // per, per * PAGE
 
@@ -684,7 +684,7 @@ def latent_attn(q_abs: torch.Tensor, cache: torch.Tensor, page_table: torch.Tens
             tile_seq, tile_q0 = ctx.query_tiles(tq)
             n_tiles = tile_seq.numel()
         _need(ctx.cu_seqlens, "latent_attn.cu_seqlens", torch.int32, (page_table.shape[0] + 1,))
-        n_splits, split_len = latent_split_plan(n_tiles * ((heads + hc - 1) // hc), max_len)
+        n_splits, split_len = latent_split_plan(n_tiles * ((heads + hc - 1) // hc), max_len, most=16)
         part = workspace("latent_attn", n_tok * heads * n_splits * (rank + 2), q_abs.device) if n_splits > 1 else None
         lib = build.variant("attn_latent_mfma", MF_LAT_DKP=(dk + 31) // 32 * 32, MF_LAT_RP=(rank + 31) // 32 * 32)
         _check(_fn("attn_latent_mfma", "mf_latent_mfma", lib)(
