@@ -10,15 +10,17 @@
 // up to multiples of 32), so queries and accumulators live in registers; the host asks for the
 // variant a model needs the first time it runs.
 //
-// A workgroup of 4 waves walks the keys in tiles of 32; wave w owns rows 16 w .. 16 w + 15.  A tile
+// A workgroup of 8 waves walks the keys in tiles of 32; waves 2 r and 2 r + 1 own rows 16 r .. 16 r + 15,
+// one for each half of the value columns (both form the rows' scores: that is the smaller of the two
+// products, and two waves on a SIMD hide each other's waits for LDS and memory).  A tile
 // is loaded into registers a tile ahead, then written to LDS twice: as it is ([key][d], for
 // q . k) and transposed ([column][key], for p . v: the matrix cores want the contracted index
 // contiguous in both operands; the transposition is 8 x 8 blocks turned in registers).  A wave
 // forms its rows' scores against the tile as S^T = K Q^T (two products of 16 keys), so that lane
 // (r, q) ends up with keys 4 q .. 4 q + 3 and 16 + 4 q .. 16 + 4 q + 3 of row r: the softmax of a
 // row stays inside its wave, and the eight probabilities of a lane are, as they lie, its share of
-// the second product's operand, O^T = V^T P^T, with the keys taken in that same order from the
-// transposed tile.  Nothing but the tile passes through LDS, and a tile costs two barriers.
+// the second product's operand, O^T = V^T P^T; the transposed tile keeps its keys in that same
+// order (`key_slot`), so a lane's eight values of a column are 16 contiguous bytes.  Nothing but the tile passes through LDS, and a tile costs two barriers.
 // 16x16x32 MFMA throughout; scores, statistics and accumulators 32-bit.
 //
 // Keys behind a sequence's last position (the rest of its last page) are written to LDS as zeros:
@@ -36,7 +38,8 @@ namespace latm {
 
 constexpr int DKP = MF_LAT_DKP, RP = MF_LAT_RP;
 constexpr int KS = DKP / 32;          // k steps of a score product
-constexpr int CT = RP / 16;           // 16-column tiles of the values
+constexpr int CT = RP / 32;           // 16-column tiles of a wave's half of the values
+constexpr int NTHR = 512;
 constexpr int M = 64, TK = 32;        // rows of a workgroup, keys of a tile
 constexpr int KSTR = DKP + 8;         // LDS row strides in elements (16 bytes of padding)
 constexpr int VSTR = TK + 8;
@@ -45,14 +48,14 @@ constexpr int VSTR = TK + 8;
 // rows, a multiple of 128 bytes apart, would all fall on the same banks
 __device__ __forceinline__ int vt_at(int col) { return col * VSTR + (col >> 3) * 8; }
 constexpr int NB8 = (DKP / 8) * (TK / 8);          // 8 x 8 blocks of a tile
-constexpr int ROUNDS = (NB8 + 255) / 256;
+constexpr int ROUNDS = (NB8 + NTHR - 1) / NTHR;
 constexpr size_t LDS_BYTES = ((size_t)TK * KSTR + (size_t)RP * VSTR + (RP / 8) * 8) * 2;
 
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 
 __device__ __forceinline__ bf16x8 as_bf16x8(u32x4 v) { return __builtin_bit_cast(bf16x8, v); }
 
-__global__ __launch_bounds__(256) void latent_mfma_kernel(
+__global__ __launch_bounds__(512) void latent_mfma_kernel(
     const bf16* __restrict__ q_abs, const bf16* __restrict__ cache, const int* __restrict__ page_table, int pt_stride,
     const int* __restrict__ positions, const int* __restrict__ cu_seqlens, const int* __restrict__ tile_seq,
     const int* __restrict__ tile_q0, bf16* __restrict__ out, float* __restrict__ part, int H, int R, int DK, int HC,
@@ -62,7 +65,8 @@ __global__ __launch_bounds__(256) void latent_mfma_kernel(
   bf16* Vt = Kt + TK * KSTR;                                // [RP][VSTR]
 
   const int lane = threadIdx.x & 63;
-  const int w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int w = wave >> 1, cw = wave & 1;         // row tile, column half
   const int r16 = lane & 15, q4 = lane >> 4;
 
   const int b = tile_seq ? tile_seq[blockIdx.x] : (int)blockIdx.x;
@@ -106,14 +110,14 @@ __global__ __launch_bounds__(256) void latent_mfma_kernel(
   // a tile ahead, in registers: 8 x 8 blocks (8 keys x 8 columns), block `blk` of a round is
   // column chunk blk % (DKP/8) of key group blk / (DKP/8)
   u32x4 pre[ROUNDS][8];
-  auto fetch = [&](int j0) {
+  auto fetch = [&](int j0, int page) {
 #pragma unroll
     for (int rd = 0; rd < ROUNDS; ++rd) {
-      const int blk = rd * 256 + (int)threadIdx.x;
+      const int blk = rd * NTHR + (int)threadIdx.x;
       const int cc = blk % (DKP / 8), kg = blk / (DKP / 8);
       const int jg = j0 + kg * 8;                  // the block's 8 keys lie in one page
       const bool live = blk < NB8 && jg <= last_pos && cc * 8 < DK;
-      const bf16* src = cache + ((size_t)(live ? pt[jg / MF_PAGE] : 0) * MF_PAGE + jg % MF_PAGE) * DK + cc * 8;
+      const bf16* src = cache + ((size_t)(live ? page : 0) * MF_PAGE + jg % MF_PAGE) * DK + cc * 8;
 #pragma unroll
       for (int k = 0; k < 8; ++k) {
         u32x4 v = {0u, 0u, 0u, 0u};
@@ -125,7 +129,7 @@ __global__ __launch_bounds__(256) void latent_mfma_kernel(
   auto stage = [&]() {
 #pragma unroll
     for (int rd = 0; rd < ROUNDS; ++rd) {
-      const int blk = rd * 256 + (int)threadIdx.x;
+      const int blk = rd * NTHR + (int)threadIdx.x;
       if (blk >= NB8) continue;
       const int cc = blk % (DKP / 8), kg = blk / (DKP / 8);
 #pragma unroll
@@ -140,18 +144,27 @@ __global__ __launch_bounds__(256) void latent_mfma_kernel(
             const unsigned a = pre[rd][2 * j2][c >> 1], bb = pre[rd][2 * j2 + 1][c >> 1];
             tv[j2] = (c & 1) ? ((a >> 16) | (bb & 0xffff0000u)) : ((a & 0xffffu) | (bb << 16));
           }
-          *reinterpret_cast<u32x4*>(Vt + vt_at(cc * 8 + c) + kg * 8) = tv;
+          // keys 8 kg .. + 3 and 8 kg + 4 .. + 7 go to the slots of two neighbouring lanes' shares
+          typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
+          bf16* vrow = Vt + vt_at(cc * 8 + c) + (kg >> 1) * 4 + (kg & 1) * 16;
+          *reinterpret_cast<u32x2*>(vrow) = u32x2{tv[0], tv[1]};
+          *reinterpret_cast<u32x2*>(vrow + 8) = u32x2{tv[2], tv[3]};
         }
       }
     }
   };
 
+  // A tile of 32 keys lies in one page.  The page number of the tile after next is asked for while
+  // the next tile's rows are on their way, so a tile waits for one trip to memory, not two in a row.
   const int tile0 = j_begin & ~(TK - 1);
-  if (tile0 < j_end) fetch(tile0);
+  auto page_of = [&](int j0) { return j0 < j_end ? pt[j0 / MF_PAGE] : 0; };
+  int page_next = page_of(tile0 + TK);
+  if (tile0 < j_end) fetch(tile0, page_of(tile0));
   for (int j0 = tile0; j0 < j_end; j0 += TK) {
     __syncthreads();                       // the tile before is no longer read
     stage();
-    if (j0 + TK < j_end) fetch(j0 + TK);
+    if (j0 + TK < j_end) fetch(j0 + TK, page_next);
+    page_next = page_of(j0 + 2 * TK);
     __syncthreads();
 
     if (!wave_live) continue;            // (uniform over the wave; the barriers above are passed by all)
@@ -193,26 +206,27 @@ __global__ __launch_bounds__(256) void latent_mfma_kernel(
     ps += __shfl_xor(ps, 32, MF_WAVE);
     l_run = l_run * corr + ps;
     m_run = m_new;
-    // O^T (columns x rows) += V^T P^T; the lane's eight keys are 4 q4 .. + 3 and 16 + 4 q4 .. + 3
+    // O^T (columns x rows) += V^T P^T; the lane's eight keys, 4 q4 .. + 3 and 16 + 4 q4 .. + 3, lie
+    // together in the transposed rows.  The accumulators are rescaled only when some row's maximum moved.
+    if (__any(corr != 1.f)) {
+#pragma unroll
+      for (int c = 0; c < CT; ++c) o[c] *= corr;
+    }
 #pragma unroll
     for (int c = 0; c < CT; ++c) {
-      o[c] *= corr;
-      const bf16* vrow = Vt + vt_at(16 * c + r16) + 4 * q4;
-      typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
-      const u32x2 lo2 = *reinterpret_cast<const u32x2*>(vrow), hi2 = *reinterpret_cast<const u32x2*>(vrow + 16);
-      const u32x4 both = {lo2[0], lo2[1], hi2[0], hi2[1]};
-      o[c] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(both), pf, o[c], 0, 0, 0);
+      const bf16x8 vf = as_bf16x8(*reinterpret_cast<const u32x4*>(Vt + vt_at(cw * (RP / 2) + 16 * c + r16) + 8 * q4));
+      o[c] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pf, o[c], 0, 0, 0);
     }
   }
 
-  // lane (r16, q4): row 16 w + r16, columns 16 c + 4 q4 + i
+  // lane (r16, q4): row 16 w + r16, columns cw RP/2 + 16 c + 4 q4 + i
   if (!row_ok) return;
   if (n_splits == 1) {
     const float inv = l_run > 0.f ? 1.0f / l_run : 0.f;
     bf16* orow = out + row_th * R;
 #pragma unroll
     for (int c = 0; c < CT; ++c) {
-      const int col = 16 * c + 4 * q4;
+      const int col = cw * (RP / 2) + 16 * c + 4 * q4;
       if (col < R) {                        // R is a multiple of 8: the four columns go together
         bf16x4 v;
 #pragma unroll
@@ -224,13 +238,13 @@ __global__ __launch_bounds__(256) void latent_mfma_kernel(
     float* prow = part + (row_th * n_splits + split) * (size_t)(R + 2);
 #pragma unroll
     for (int c = 0; c < CT; ++c) {
-      const int col = 16 * c + 4 * q4;
+      const int col = cw * (RP / 2) + 16 * c + 4 * q4;
       if (col < R) {
 #pragma unroll
         for (int i = 0; i < 4; ++i) prow[col + i] = o[c][i];
       }
     }
-    if (q4 == 0) { prow[R] = m_run; prow[R + 1] = l_run; }
+    if (q4 == 0 && cw == 0) { prow[R] = m_run; prow[R + 1] = l_run; }
   }
 }
 
@@ -296,7 +310,7 @@ MF_API int mf_latent_mfma(const void* q_abs, const void* cache, const int* page_
     raised = true;
   }
   dim3 grid(n_tiles, (H + HC - 1) / HC, n_splits);
-  latent_mfma_kernel<<<grid, 256, LDS_BYTES, stream>>>(
+  latent_mfma_kernel<<<grid, NTHR, LDS_BYTES, stream>>>(
       (const bf16*)q_abs, (const bf16*)cache, page_table, pt_stride, positions, cu_seqlens, tile_seq, tile_q0,
       (bf16*)out, part, H, R, DK, HC, TQ, scale, window, n_splits, split_len);
   int rc = mf_launch_status();

@@ -63,7 +63,36 @@ def variant(base: str, **sizes: int) -> str:
         DEFINES[name] = DEFINES.get(base, []) + [f"-D{k}={int(v)}" for k, v in sorted(sizes.items())]
         if base in HEADERS:
             HEADERS[name] = HEADERS[base]
+        _note_variant(base, sizes)
     return name
+
+
+def _variants_file() -> str:
+    return os.path.join(lib_dir(), "variants.txt")
+
+
+def _note_variant(base: str, sizes: Dict[str, int]) -> None:
+    """Keeps the variants that were ever asked for beside the built files, so that `build_all`
+    builds them again with the rest."""
+    line = base + " " + " ".join(f"{k}={int(v)}" for k, v in sorted(sizes.items()))
+    try:
+        have = open(_variants_file()).read().splitlines() if os.path.exists(_variants_file()) else []
+        if line not in have:
+            with open(_variants_file(), "a") as f:
+                f.write(line + "\n")
+    except OSError:
+        pass
+
+
+def known_variants() -> List[str]:
+    """Registers the variants listed beside the built files and returns their names."""
+    names = []
+    if os.path.exists(_variants_file()):
+        for line in open(_variants_file()).read().splitlines():
+            parts = line.split()
+            if parts and parts[0] in LIBRARIES:
+                names.append(variant(parts[0], **{k: int(v) for k, v in (p.split("=") for p in parts[1:])}))
+    return names
 
 
 def _hipcc() -> str:
@@ -170,7 +199,9 @@ def compile_library(name: str, quiet: bool = False) -> str:
 
 
 def build_all(force: bool = True, jobs: int = 4) -> List[str]:
-    """Compiles every library (always, when `force`), a few at a time."""
+    """Compiles every library and every sized variant asked for before (always, when `force`), a few
+    at a time."""
+    known_variants()
     names = [n for n in LIBRARIES if force or not is_current(n)]
     errors, lock = [], threading.Lock()
     pending = list(names)

@@ -684,7 +684,7 @@ def latent_attn(q_abs: torch.Tensor, cache: torch.Tensor, page_table: torch.Tens
             tile_seq, tile_q0 = ctx.query_tiles(tq)
             n_tiles = tile_seq.numel()
         _need(ctx.cu_seqlens, "latent_attn.cu_seqlens", torch.int32, (page_table.shape[0] + 1,))
-        n_splits, split_len = latent_split_plan(n_tiles * ((heads + hc - 1) // hc), max_len, most=16)
+        n_splits, split_len = latent_split_plan(n_tiles * ((heads + hc - 1) // hc), max_len, target_blocks=2 * cu_count(), most=32)
         part = workspace("latent_attn", n_tok * heads * n_splits * (rank + 2), q_abs.device) if n_splits > 1 else None
         lib = build.variant("attn_latent_mfma", MF_LAT_DKP=(dk + 31) // 32 * 32, MF_LAT_RP=(rank + 31) // 32 * 32)
         _check(_fn("attn_latent_mfma", "mf_latent_mfma", lib)(
