@@ -72,6 +72,8 @@ def parse():
                     help="instead of the default workload: prefill and decode of this design at a few layer sizes "
                          "beside the Qwen2 decoder of the same width, depth and feed-forward size, kernel by kernel")
     ap.add_argument("--design-sizes", default="small,medium", help="which of the design's sizes to run")
+    ap.add_argument("--design-model", default="tabezen", choices=["tabezen", "qwen2"],
+                    help="with --design and --only: which of the two models runs the one part (for profiles)")
     return ap.parse_args()
 
 
@@ -337,6 +339,18 @@ def attention_rooflines(size, a, point, design):
 def run_design(a) -> int:
     dtype = {"bf16": "bfloat16", "fp32": "float32"}[a.dtype]
     elem = 2 if a.dtype == "bf16" else 4
+    if a.only:                               # one part of one model at the first size, for profiles
+        from minfer_amd import LLM
+        size = DESIGN_SIZES[a.design_sizes.split(",")[0]]
+        cfg = tabezen_config(**size) if a.design_model == "tabezen" else qwen2_like(**size)
+        eng = LLM(config=cfg, random_weights=True, weight_seed=0, dtype=dtype, n_ctx=a.context, n_slots=a.batch).engine
+        if a.only == "decode":
+            r = run_decode(eng, cfg, a.batch, a.prompt_max, a.steps, a.warmup, not a.no_graph, elem, bytes_fn=lambda *_: 0.0)
+            print(f"{a.design_model} decode batch {a.batch}: {r['tok_s']:.1f} tok/s, {r['ms']:.3f} ms/step")
+        else:
+            s = run_prefill(eng, cfg, a.prefill_tokens)
+            print(f"{a.design_model} prefill {a.prefill_tokens} tokens: {s * 1e3:.2f} ms, {a.prefill_tokens / s:.0f} tok/s")
+        return 0
     out = {"design": a.design, "dtype": a.dtype, "data": "synthetic", "batch": a.batch, "prompt_max": a.prompt_max,
            "prefill_tokens": a.prefill_tokens, "steps": a.steps, "warmup": a.warmup, "sizes": {}}
     for name in a.design_sizes.split(","):

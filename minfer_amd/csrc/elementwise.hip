@@ -129,23 +129,51 @@ __global__ __launch_bounds__(256) void group_rmsnorm_kernel(const float* x,
     const int tpg = 256 / groups;                  // threads of a group: a power of two
     const int g = threadIdx.x / tpg, tl = threadIdx.x % tpg;
     const int lo = g * part;
+    auto group_total = [&](float ss) {
+#pragma unroll
+      for (int off = 1; off < 64; off <<= 1)
+        if (off < tpg) ss += __shfl_xor(ss, off, MF_WAVE);
+      if (tpg > 64) {                              // the group's waves meet in LDS
+        const int wv = threadIdx.x >> 6;
+        if ((threadIdx.x & 63) == 0) scratch[wv] = ss;
+        __syncthreads();
+        const int w0 = (wv / (tpg / 64)) * (tpg / 64);
+        ss = 0.f;
+        for (int k = 0; k < tpg / 64; ++k) ss += scratch[w0 + k];
+      }
+      return ss;
+    };
+    constexpr int KEEP = 16;
+    if (d % 256 == 0 && d <= 256 * KEEP) {         // a thread's d / 256 values, gains and old sums in one trip
+      const int ept = d / 256;
+      float xv[KEEP], gv[KEEP], ov[KEEP];
+      float ss = 0.f;
+#pragma unroll
+      for (int k = 0; k < KEEP; ++k) {
+        const int i = lo + tl + k * tpg;
+        xv[k] = k < ept ? xr[i] : 0.f;
+        gv[k] = (k < ept && w) ? w[i] : 1.0f;
+        ov[k] = (ADD && k < ept) ? to_f32(o[i]) : 0.f;
+        ss = fmaf(xv[k], xv[k], ss);
+      }
+      const float scale = 1.0f / sqrtf(group_total(ss) / (float)part + eps);
+#pragma unroll
+      for (int k = 0; k < KEEP; ++k) {
+        if (k < ept) {
+          const int i = lo + tl + k * tpg;
+          const float y = xv[k] * scale * gv[k] + ov[k];
+          o[i] = from_f32<OT>(y);
+          if (co) co[i] = (bf16)y;
+        }
+      }
+      return;
+    }
     float ss = 0.f;
     for (int i = tl; i < part; i += tpg) {
       const float v = xr[lo + i];
       ss = fmaf(v, v, ss);
     }
-#pragma unroll
-    for (int off = 1; off < 64; off <<= 1)
-      if (off < tpg) ss += __shfl_xor(ss, off, MF_WAVE);
-    if (tpg > 64) {                                // the group's waves meet in LDS
-      const int wv = threadIdx.x >> 6;
-      if ((threadIdx.x & 63) == 0) scratch[wv] = ss;
-      __syncthreads();
-      const int w0 = (wv / (tpg / 64)) * (tpg / 64);
-      ss = 0.f;
-      for (int k = 0; k < tpg / 64; ++k) ss += scratch[w0 + k];
-    }
-    const float scale = 1.0f / sqrtf(ss / (float)part + eps);
+    const float scale = 1.0f / sqrtf(group_total(ss) / (float)part + eps);
     for (int i = tl; i < part; i += tpg) {
       float y = xr[lo + i] * scale * (w ? w[lo + i] : 1.0f);
       if (ADD) y += to_f32(o[lo + i]);

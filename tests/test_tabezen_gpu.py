@@ -51,7 +51,8 @@ def compare(rows, ref, dtype, what, loosen=1.0, f32_abs=F32_ABS):
 
 
 # ------------------------------------------------------------------ kernels alone
-@pytest.mark.parametrize("d, groups", [(96, 3), (200, 1), (1028, 4), (64, 64)])
+@pytest.mark.parametrize("d, groups", [(96, 3), (200, 1), (1028, 4), (64, 64), (512, 4), (2048, 2), (4096, 1), (256, 256),
+                                       (8192, 8)])
 def test_group_rmsnorm_kernel(d, groups):
     from minfer_amd.kernels import ops
     x, w = rnd(7, d, seed=1, scale=3.0), rnd(d, seed=2) + 1
