@@ -21,7 +21,7 @@
 
 // ------------------------------------------------------------------ preparation
 // proj: 32-bit rows [q: H (DN + DR) | dkv: R + DR | gate: H] at the given offsets of a row of
-// `ld` floats.  One block per token.
+// `ld` floats.  Two blocks per token: one for the cached row, one for the queries and gates.
 template <typename OT>
 __global__ __launch_bounds__(256) void latent_prep_kernel(
     const float* __restrict__ proj, int ld, int off_dkv, int off_gate, const float* __restrict__ cw, float eps,
@@ -36,13 +36,14 @@ __global__ __launch_bounds__(256) void latent_prep_kernel(
   const int DK = R + DR, half = rd >> 1;
   const float* c_t = cs + (size_t)pos * half;
   const float* s_t = sn + (size_t)pos * half;
-  // the latent: x / sqrt(mean(x^2) + eps) * w
-  const float* dkv = row + off_dkv;
-  float ss = 0.f;
-  for (int i = threadIdx.x; i < R; i += 256) ss = fmaf(dkv[i], dkv[i], ss);
-  ss = block_sum<256>(ss, scratch);
-  const float inv = 1.0f / sqrtf(ss / (float)R + eps);
-  if (write_cache) {
+  if (blockIdx.y == 0) {
+    if (!write_cache) return;
+    // the latent: x / sqrt(mean(x^2) + eps) * w
+    const float* dkv = row + off_dkv;
+    float ss = 0.f;
+    for (int i = threadIdx.x; i < R; i += 256) ss = fmaf(dkv[i], dkv[i], ss);
+    ss = block_sum<256>(ss, scratch);
+    const float inv = 1.0f / sqrtf(ss / (float)R + eps);
     const int page = page_table[(size_t)seq_of_tok[t] * pt_stride + pos / MF_PAGE];
     OT* dst = cache + ((size_t)page * MF_PAGE + pos % MF_PAGE) * DK;
     for (int i = threadIdx.x; i < R; i += 256) dst[i] = from_f32<OT>(dkv[i] * inv * cw[i]);
@@ -58,6 +59,7 @@ __global__ __launch_bounds__(256) void latent_prep_kernel(
       }
       dst[R + i] = from_f32<OT>(v);
     }
+    return;
   }
   // queries: plain part as it is, rotated part behind the R columns the absorption will fill
   const int DQ = DN + DR;
@@ -90,11 +92,11 @@ MF_API int mf_latent_prep(const float* proj, int ld, int off_dkv, int off_gate, 
   if (n_tok <= 0) return 0;
   if (rd < 0 || rd > DR || (rd & 1) || H < 1 || DN < 1 || R < 1) return (int)hipErrorInvalidValue;
   if (is_bf16)
-    latent_prep_kernel<bf16><<<n_tok, 256, 0, stream>>>(proj, ld, off_dkv, off_gate, cw, eps, cs, sn, rd, positions,
+    latent_prep_kernel<bf16><<<dim3(n_tok, 2), 256, 0, stream>>>(proj, ld, off_dkv, off_gate, cw, eps, cs, sn, rd, positions,
                                                          seq_of_tok, page_table, pt_stride, (bf16*)cache,
                                                          (bf16*)q_plain, (bf16*)q_abs, gate, H, DN, DR, R, write_cache);
   else
-    latent_prep_kernel<float><<<n_tok, 256, 0, stream>>>(proj, ld, off_dkv, off_gate, cw, eps, cs, sn, rd, positions,
+    latent_prep_kernel<float><<<dim3(n_tok, 2), 256, 0, stream>>>(proj, ld, off_dkv, off_gate, cw, eps, cs, sn, rd, positions,
                                                           seq_of_tok, page_table, pt_stride, (float*)cache,
                                                           (float*)q_plain, (float*)q_abs, gate, H, DN, DR, R,
                                                           write_cache);

@@ -10,10 +10,11 @@
 // up to multiples of 32), so queries and accumulators live in registers; the host asks for the
 // variant a model needs the first time it runs.
 //
-// A workgroup of 8 waves walks the keys in tiles of 32; waves 2 r and 2 r + 1 own rows 16 r .. 16 r + 15,
+// A workgroup of 8 waves walks the keys in tiles of 32 (two tiles ahead of the products, their rows
+// are on their way from the cache into registers); waves 2 r and 2 r + 1 own rows 16 r .. 16 r + 15,
 // one for each half of the value columns (both form the rows' scores: that is the smaller of the two
 // products, and two waves on a SIMD hide each other's waits for LDS and memory).  A tile
-// is loaded into registers a tile ahead, then written to LDS twice: as it is ([key][d], for
+// is written to LDS twice: as it is ([key][d], for
 // q . k) and transposed ([column][key], for p . v: the matrix cores want the contracted index
 // contiguous in both operands; the transposition is 8 x 8 blocks turned in registers).  A wave
 // forms its rows' scores against the tile as S^T = K Q^T (two products of 16 keys), so that lane
@@ -69,18 +70,22 @@ __global__ __launch_bounds__(512) void latent_mfma_kernel(
   const int w = wave >> 1, cw = wave & 1;         // row tile, column half
   const int r16 = lane & 15, q4 = lane >> 4;
 
+  // Without `cu_seqlens` every sequence brings one token (tile i is token i of sequence i): the
+  // token's position and its queries are asked for at once.
+  const bool single = cu_seqlens == nullptr;
   const int b = tile_seq ? tile_seq[blockIdx.x] : (int)blockIdx.x;
   const int q0 = tile_q0 ? tile_q0[blockIdx.x] : 0;
   const int h0 = blockIdx.y * HC;
   const int hcount = min(HC, H - h0);
   const int split = blockIdx.z;
-  const int t_first = cu_seqlens[b] + q0;
-  const int n_here = min(TQ, cu_seqlens[b + 1] - t_first);
   const int* pt = page_table + (size_t)b * pt_stride;
+  const int early = split * split_len;                      // the split's first key, unless a window cuts it
+  const int t_first = single ? b : cu_seqlens[b] + q0;
+  const int n_here = single ? 1 : min(TQ, cu_seqlens[b + 1] - t_first);
   const int first_pos = positions[t_first];
   const int last_pos = first_pos + n_here - 1;              // new tokens of a sequence are consecutive
   const int lo_all = window > 0 ? max(0, first_pos - window + 1) : 0;
-  const int j_begin = max(lo_all, split * split_len);
+  const int j_begin = max(lo_all, early);
   const int j_end = min(last_pos + 1, (split + 1) * split_len);
 
   // this lane's row, its position and query
@@ -107,15 +112,16 @@ __global__ __launch_bounds__(512) void latent_mfma_kernel(
   for (int c = 0; c < CT; ++c) o[c] = floatx4{0.f, 0.f, 0.f, 0.f};
   float m_run = -INFINITY, l_run = 0.f;
 
-  // a tile ahead, in registers: 8 x 8 blocks (8 keys x 8 columns), block `blk` of a round is
-  // column chunk blk % (DKP/8) of key group blk / (DKP/8)
-  u32x4 pre[ROUNDS][8];
-  auto fetch = [&](int j0, int page) {
+  // two tiles ahead, in registers: 8 x 8 blocks (8 keys x 8 columns), block `blk` of a round is
+  // column chunk blk % (DKP/8) of key group blk / (DKP/8).  A tile of 32 keys lies in one page.
+  u32x4 pre_a[ROUNDS][8], pre_b[ROUNDS][8];
+  auto fetch = [&](u32x4 (&pre)[ROUNDS][8], int j0) {
+    const int page = j0 <= last_pos ? pt[j0 / MF_PAGE] : 0;
 #pragma unroll
     for (int rd = 0; rd < ROUNDS; ++rd) {
       const int blk = rd * NTHR + (int)threadIdx.x;
       const int cc = blk % (DKP / 8), kg = blk / (DKP / 8);
-      const int jg = j0 + kg * 8;                  // the block's 8 keys lie in one page
+      const int jg = j0 + kg * 8;
       const bool live = blk < NB8 && jg <= last_pos && cc * 8 < DK;
       const bf16* src = cache + ((size_t)(live ? page : 0) * MF_PAGE + jg % MF_PAGE) * DK + cc * 8;
 #pragma unroll
@@ -126,7 +132,7 @@ __global__ __launch_bounds__(512) void latent_mfma_kernel(
       }
     }
   };
-  auto stage = [&]() {
+  auto stage = [&](const u32x4 (&pre)[ROUNDS][8]) {
 #pragma unroll
     for (int rd = 0; rd < ROUNDS; ++rd) {
       const int blk = rd * NTHR + (int)threadIdx.x;
@@ -154,20 +160,8 @@ __global__ __launch_bounds__(512) void latent_mfma_kernel(
     }
   };
 
-  // A tile of 32 keys lies in one page.  The page number of the tile after next is asked for while
-  // the next tile's rows are on their way, so a tile waits for one trip to memory, not two in a row.
-  const int tile0 = j_begin & ~(TK - 1);
-  auto page_of = [&](int j0) { return j0 < j_end ? pt[j0 / MF_PAGE] : 0; };
-  int page_next = page_of(tile0 + TK);
-  if (tile0 < j_end) fetch(tile0, page_of(tile0));
-  for (int j0 = tile0; j0 < j_end; j0 += TK) {
-    __syncthreads();                       // the tile before is no longer read
-    stage();
-    if (j0 + TK < j_end) fetch(j0 + TK, page_next);
-    page_next = page_of(j0 + 2 * TK);
-    __syncthreads();
-
-    if (!wave_live) continue;            // (uniform over the wave; the barriers above are passed by all)
+  auto compute = [&](int j0) {
+    if (!wave_live) return;              // (uniform over the wave)
     // scores: S^T (keys x rows), keys 0..15 and 16..31 of the tile
     floatx4 s2[2] = {floatx4{0.f, 0.f, 0.f, 0.f}, floatx4{0.f, 0.f, 0.f, 0.f}};
 #pragma unroll
@@ -216,6 +210,24 @@ __global__ __launch_bounds__(512) void latent_mfma_kernel(
     for (int c = 0; c < CT; ++c) {
       const bf16x8 vf = as_bf16x8(*reinterpret_cast<const u32x4*>(Vt + vt_at(cw * (RP / 2) + 16 * c + r16) + 8 * q4));
       o[c] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pf, o[c], 0, 0, 0);
+    }
+  };
+
+  const int tile0 = j_begin & ~(TK - 1);
+  if (tile0 < j_end) fetch(pre_a, tile0);
+  if (tile0 + TK < j_end) fetch(pre_b, tile0 + TK);
+  for (int j0 = tile0; j0 < j_end; j0 += 2 * TK) {
+    __syncthreads();                       // the tile before is no longer read
+    stage(pre_a);
+    if (j0 + 2 * TK < j_end) fetch(pre_a, j0 + 2 * TK);
+    __syncthreads();
+    compute(j0);
+    if (j0 + TK < j_end) {                 // (uniform over the workgroup)
+      __syncthreads();
+      stage(pre_b);
+      if (j0 + 3 * TK < j_end) fetch(pre_b, j0 + 3 * TK);
+      __syncthreads();
+      compute(j0 + TK);
     }
   }
 
@@ -290,8 +302,8 @@ MF_API int mf_latent_mfma_sizes(int* dkp, int* rp) {
   return 0;
 }
 
-// tile_seq / tile_q0: the workgroups' (sequence, first new token) pairs, n_tiles of them; null for
-// a step in which every sequence brings one token (tile i is sequence i).
+// tile_seq / tile_q0: the workgroups' (sequence, first new token) pairs, n_tiles of them; null, and
+// cu_seqlens null as well, for a step in which every sequence brings one token (tile i is sequence i).
 MF_API int mf_latent_mfma(const void* q_abs, const void* cache, const int* page_table, int pt_stride,
                           const int* positions, const int* cu_seqlens, const int* tile_seq, const int* tile_q0,
                           int n_tiles, void* out, float* part, int n_tok, int H, int R, int DK, int HC, int TQ,

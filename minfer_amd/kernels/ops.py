@@ -678,17 +678,18 @@ def latent_attn(q_abs: torch.Tensor, cache: torch.Tensor, page_table: torch.Tens
         hc = min(heads, LATENT_MFMA_ROWS)
         tq = LATENT_MFMA_ROWS // hc
         if ctx.all_decode:
-            tile_seq = tile_q0 = None
+            tile_seq = tile_q0 = cu = None
             n_tiles = n_tok
         else:
             tile_seq, tile_q0 = ctx.query_tiles(tq)
             n_tiles = tile_seq.numel()
-        _need(ctx.cu_seqlens, "latent_attn.cu_seqlens", torch.int32, (page_table.shape[0] + 1,))
+            cu = ctx.cu_seqlens
+            _need(cu, "latent_attn.cu_seqlens", torch.int32, (page_table.shape[0] + 1,))
         n_splits, split_len = latent_split_plan(n_tiles * ((heads + hc - 1) // hc), max_len, target_blocks=2 * cu_count(), most=32)
         part = workspace("latent_attn", n_tok * heads * n_splits * (rank + 2), q_abs.device) if n_splits > 1 else None
         lib = build.variant("attn_latent_mfma", MF_LAT_DKP=(dk + 31) // 32 * 32, MF_LAT_RP=(rank + 31) // 32 * 32)
         _check(_fn("attn_latent_mfma", "mf_latent_mfma", lib)(
-            _ptr(q_abs), _ptr(cache), _ptr(page_table), page_table.shape[1], _ptr(positions), _ptr(ctx.cu_seqlens),
+            _ptr(q_abs), _ptr(cache), _ptr(page_table), page_table.shape[1], _ptr(positions), _ptr(cu),
             _ptr(tile_seq), _ptr(tile_q0), n_tiles, _ptr(out), _ptr(part), n_tok, heads, rank, dk, hc, tq, float(scale),
             int(window), n_splits, split_len, _stream()), "latent_attn_mfma")
         return
