@@ -38,10 +38,19 @@
 
 namespace {
 
-enum { EPI_F32 = 0, EPI_ACC_F32 = 1, EPI_BF16 = 2, EPI_SWIGLU = 3 };
+// EPI_XIELU: bfloat16 output of the xIELU activation of (sum + bias); the activation's two constants
+// (a_pos, a_neg: z > 0 -> a_pos z^2 + z/2, else a_neg (e^z - 1 - z) + z/2) stand behind the N biases.
+enum { EPI_F32 = 0, EPI_ACC_F32 = 1, EPI_BF16 = 2, EPI_SWIGLU = 3, EPI_XIELU = 4 };
 
-__device__ __forceinline__ void store_out(void* C, int ldc, int m, int n, float v, int epi) {
-  if (epi == EPI_BF16) {
+__device__ __forceinline__ float xielu_f(float z, float a_pos, float a_neg) {
+  return z > 0.f ? fmaf(a_pos * z, z, 0.5f * z) : fmaf(a_neg, expm1f(z) - z, 0.5f * z);
+}
+
+__device__ __forceinline__ void store_out(void* C, int ldc, int m, int n, float v, int epi,
+                                          const float* __restrict__ bias = nullptr, int N = 0) {
+  if (epi == EPI_XIELU) {
+    ((bf16*)C)[(size_t)m * ldc + n] = (bf16)xielu_f(v, bias[N], bias[N + 1]);
+  } else if (epi == EPI_BF16) {
     ((bf16*)C)[(size_t)m * ldc + n] = (bf16)v;
   } else {
     float* c = (float*)C + (size_t)m * ldc + n;
@@ -112,7 +121,7 @@ __device__ __forceinline__ void tile_epilogue(floatx16 (&acc)[TM][TN], const flo
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
         const int m = m0 + wm + i * 32 + (r >> 2) * 8 + (lane >> 5) * 4 + (r & 3);
-        if (m < M) store_out(C, ldc, m, n, acc[i][j][r] + b, epi);
+        if (m < M) store_out(C, ldc, m, n, acc[i][j][r] + b, epi, bias, N);
       }
     }
 }
@@ -623,7 +632,7 @@ __global__ __launch_bounds__(512) void skinny_kernel(const bf16* __restrict__ A,
       if (part) {
         part[((size_t)blockIdx.y * M + m) * N + n_row] = acc[i][r];
       } else {
-        store_out(C, ldc, m, n_row, acc[i][r] + (bias ? bias[n_row] : 0.f), epi);
+        store_out(C, ldc, m, n_row, acc[i][r] + (bias ? bias[n_row] : 0.f), epi, bias, N);
       }
     }
 }
@@ -703,7 +712,7 @@ __global__ __launch_bounds__(512) void skinny_ring_kernel(const bf16* __restrict
     for (int m = tid >> 7; m < M; m += 4) part[((size_t)blockIdx.y * M + m) * N + n] = ot[m * SR_LD + c];
   } else {
     const float b = bias ? bias[n] : 0.f;
-    for (int m = tid >> 7; m < M; m += 4) store_out(C, ldc, m, n, ot[m * SR_LD + c] + b, epi);
+    for (int m = tid >> 7; m < M; m += 4) store_out(C, ldc, m, n, ot[m * SR_LD + c] + b, epi, bias, N);
   }
 }
 
@@ -815,7 +824,7 @@ __global__ __launch_bounds__(NW * 64) void skinny16_kernel(const bf16* __restric
       float v = 0.f;
 #pragma unroll
       for (int w = 0; w < NW; ++w) v += red[w][j][lane][r];
-      store_out(C, ldc, m, n, v + b, epi);
+      store_out(C, ldc, m, n, v + b, epi, bias, N);
     }
   }
 }
@@ -1077,7 +1086,7 @@ __global__ __launch_bounds__(NW * 64) void rolling16_kernel(const bf16* __restri
     for (int ww = 0; ww < NW; ++ww) v += red[ww][e_m][e_c];
     if (epi == EPI_ACC_F32) v += c_old;
     if (epi == EPI_ACC_F32) ((float*)C)[(size_t)e_m * ldc + e_n] = v;
-    else store_out(C, ldc, e_m, e_n, v, epi);
+    else store_out(C, ldc, e_m, e_n, v, epi, bias, N);
     if (fused.out_g) {
       fused.out_xg[(size_t)e_m * ldc + e_n] = (bf16)(v * e_g);
       sq = v * v;
@@ -1396,7 +1405,7 @@ __global__ __launch_bounds__(NW * 64) void stationary16_kernel(const void* __res
         v += (bias ? e_bias : 0.f);
         if (epi == EPI_ACC_F32) v += c_old;
         if (epi == EPI_ACC_F32) ((float*)C)[(size_t)e_m * ldc + e_n] = v;
-        else store_out(C, ldc, e_m, e_n, v, epi);
+        else store_out(C, ldc, e_m, e_n, v, epi, bias, N);
         if (fused.out_g) {
           fused.out_xg[(size_t)e_m * ldc + e_n] = (bf16)(v * e_g);
           sq = fmaf(v, v, sq);
@@ -1609,7 +1618,7 @@ __global__ __launch_bounds__(512) void panel_kernel(const bf16* __restrict__ A, 
         const int col = u0 * 32 + c;
         if (c < cnt * 16 && col < N) {
           const float b = bias ? bias[col] : 0.f;
-          for (int m = tid >> 8; m < M; m += 2) store_out(C, ldc, m, col, ot[m * OT_LD + c] * rfac[m] + b, epi);
+          for (int m = tid >> 8; m < M; m += 2) store_out(C, ldc, m, col, ot[m * OT_LD + c] * rfac[m] + b, epi, bias, N);
         }
       }
     }
@@ -1673,7 +1682,9 @@ __global__ __launch_bounds__(256) void skinny_reduce_kernel(const float* __restr
   float v = 0.f;                 // the output's new value (0 beyond the row's end)
   if (n < N) {
     v = sum_of_parts(part, stride, (size_t)m * N + n, splits) * rf + (bias ? bias[n] : 0.f);
-    if (epi == EPI_BF16) {
+    if (epi == EPI_XIELU) {
+      ((bf16*)C)[(size_t)m * ldc + n] = (bf16)xielu_f(v, bias[N], bias[N + 1]);
+    } else if (epi == EPI_BF16) {
       ((bf16*)C)[(size_t)m * ldc + n] = (bf16)v;
     } else {
       float* c = (float*)C + (size_t)m * ldc + n;
@@ -1731,7 +1742,12 @@ __global__ __launch_bounds__(256) void skinny_reduce4_kernel(const float* __rest
     const float rf = ffac[0];
     const float4 b = bias ? *reinterpret_cast<const float4*>(bias + n) : float4{0.f, 0.f, 0.f, 0.f};
     v = float4{v.x * rf + b.x, v.y * rf + b.y, v.z * rf + b.z, v.w * rf + b.w};
-    if (epi == EPI_BF16) {
+    if (epi == EPI_XIELU) {
+      const float ap = bias[N], an = bias[N + 1];
+      bf16* c = (bf16*)C + (size_t)m * ldc + n;
+      c[0] = (bf16)xielu_f(v.x, ap, an); c[1] = (bf16)xielu_f(v.y, ap, an);
+      c[2] = (bf16)xielu_f(v.z, ap, an); c[3] = (bf16)xielu_f(v.w, ap, an);
+    } else if (epi == EPI_BF16) {
       bf16* c = (bf16*)C + (size_t)m * ldc + n;
       c[0] = (bf16)v.x; c[1] = (bf16)v.y; c[2] = (bf16)v.z; c[3] = (bf16)v.w;
     } else {
@@ -1888,7 +1904,7 @@ TilePlan plan_tiles(int M, int N, int K, bool dma_ok, int epi, int n_cu) {
   const long cu = n_cu > 0 ? n_cu : 1;
   const long nkt = (K + 63) / 64, chunks = (K + 255) / 256;
   const double mn = (double)M * (double)N;
-  const double epi_us = (epi == EPI_ACC_F32 ? 8. : epi == EPI_F32 ? 4. : epi == EPI_BF16 ? 2. : 1.) * mn / 4e6;
+  const double epi_us = (epi == EPI_ACC_F32 ? 8. : epi == EPI_F32 ? 4. : (epi == EPI_BF16 || epi == EPI_XIELU) ? 2. : 1.) * mn / 4e6;
   const double start_us = 12.;
   auto tiles = [&](int bm, int bn) { return (long)((M + bm - 1) / bm) * ((N + bn - 1) / bn); };
   auto cut = [&](long parts, int& splits, int& per) {          // K in `parts` runs of whole chunks of 256
@@ -1966,7 +1982,7 @@ SkinnyChoice skinny_choice(int M, int N, int K, bool aligned, int epi, int split
 MF_API int mf_gemm_bf16(const void* A, int lda, const void* W, int ldw, const float* bias, void* C,
                         int ldc, int M, int N, int K, int epi, int variant, hipStream_t stream) {
   if (M <= 0 || N <= 0) return 0;
-  if (K <= 0 || lda < K || ldw < K || epi < 0 || epi > 3) return (int)hipErrorInvalidValue;
+  if (K <= 0 || lda < K || ldw < K || epi < 0 || epi > EPI_XIELU || (epi == EPI_XIELU && !bias)) return (int)hipErrorInvalidValue;
   if (epi == EPI_SWIGLU ? (N % 64 != 0 || ldc > N / 2 || ldc <= N / 2 - 32 || bias) : ldc < N)
     return (int)hipErrorInvalidValue;
   const int vec_ok = (lda % 8 == 0) && (ldw % 8 == 0) && ((uintptr_t)A % 16 == 0) &&
@@ -2008,7 +2024,7 @@ MF_API int mf_gemm_bf16_splitk(const void* A, int lda, const void* W, int ldw, c
                                int ldc, float* part, int M, int N, int K, int splits, int k_per_split,
                                int epi, int variant, hipStream_t stream) {
   if (M <= 0 || N <= 0) return 0;
-  if (K <= 0 || lda < K || ldw < K || epi < 0 || epi > 3 || splits < 2 || !part || k_per_split % 64 != 0 ||
+  if (K <= 0 || lda < K || ldw < K || epi < 0 || epi > EPI_XIELU || (epi == EPI_XIELU && !bias) || splits < 2 || !part || k_per_split % 64 != 0 ||
       (long)splits * k_per_split < K || (long)(splits - 1) * k_per_split >= K)
     return (int)hipErrorInvalidValue;
   if (epi == EPI_SWIGLU ? (N % 64 != 0 || ldc > N / 2 || ldc <= N / 2 - 32 || bias) : ldc < N)
@@ -2064,7 +2080,7 @@ static int skinny_product(const void* A, int lda, const void* W, const void* Wt,
                           void* C, int ldc, float* part, int M, int N, int K, int splits, int k_per_split, int epi,
                           const FusedNorm& fused, hipStream_t stream) {
   if (M <= 0 || N <= 0) return 0;
-  if (M > 64 || K <= 0 || lda < K || ldw < K || epi < 0 || epi > 3 || splits < 1 ||
+  if (M > 64 || K <= 0 || lda < K || ldw < K || epi < 0 || epi > EPI_XIELU || (epi == EPI_XIELU && !bias) || splits < 1 ||
       k_per_split % KC != 0 || (long)splits * k_per_split < K || (splits > 1 && !part))
     return (int)hipErrorInvalidValue;
   if (epi == EPI_SWIGLU ? (N % 64 != 0 || ldc > N / 2 || ldc <= N / 2 - 32 || bias || (M > 16 && !part))
@@ -2143,7 +2159,7 @@ MF_API int mf_gemm_bf16_normed(const float* x, int ldx, const int* row_idx, cons
                                const void* W, const void* Wt, int ldw, const float* bias, void* C, int ldc, int M,
                                int N, int K, int epi, hipStream_t stream) {
   if (M <= 0 || N <= 0) return 0;
-  if (K <= 0 || epi < 0 || epi > EPI_SWIGLU) return (int)hipErrorInvalidValue;
+  if (K <= 0 || epi < 0 || epi > EPI_XIELU || (epi == EPI_XIELU && !bias)) return (int)hipErrorInvalidValue;
   if (ldx % 4 != 0 || ldw % 8 != 0 || (uintptr_t)x % 16 != 0 || (uintptr_t)g % 16 != 0 || (uintptr_t)W % 16 != 0)
     return MF_NOT_BUILT;
   const NormArgs norm{g, row_idx, eps};
@@ -2155,7 +2171,7 @@ MF_API int mf_gemm_bf16_normed(const float* x, int ldx, const int* row_idx, cons
 // for mf_gemm_bf16_splitk with out[1] splits of out[2] of K each.  `aligned`: 16-byte aligned
 // operands with row strides and K in multiples of 8.
 MF_API int mf_gemm_bf16_tile_plan(int M, int N, int K, int aligned, int epi, int n_cu, int* out) {
-  if (!out || M <= 0 || N <= 0 || K <= 0 || epi < 0 || epi > 3 || n_cu <= 0) return (int)hipErrorInvalidValue;
+  if (!out || M <= 0 || N <= 0 || K <= 0 || epi < 0 || epi > EPI_XIELU || n_cu <= 0) return (int)hipErrorInvalidValue;
   const bool dma_ok = aligned && K % DMA_BK == 0 && (size_t)M * K * 2 < (1ull << 32) && (size_t)N * K * 2 < (1ull << 32);
   const TilePlan plan = plan_tiles(M, N, K, dma_ok, epi, n_cu);
   out[0] = plan.variant;
@@ -2171,7 +2187,7 @@ MF_API int mf_gemm_bf16_tile_plan(int M, int N, int K, int aligned, int epi, int
 // such kernel": norm and product run one after the other); `n_cu`: compute units of the device.
 MF_API int mf_gemm_bf16_plan(int M, int N, int K, int aligned, int epi, int splits, int k_per_split,
                              int normed, int n_cu, char* name, int cap) {
-  if (!name || cap < 48 || M <= 0 || N <= 0 || K <= 0 || epi < 0 || epi > 3 || n_cu <= 0) return (int)hipErrorInvalidValue;
+  if (!name || cap < 48 || M <= 0 || N <= 0 || K <= 0 || epi < 0 || epi > EPI_XIELU || n_cu <= 0) return (int)hipErrorInvalidValue;
   const char* what = "";
   if (normed) {
     what = (aligned && stationary_takes(M, N, K, epi, true)) ? "stationary16_kernel(norm)" : "";

@@ -19,7 +19,7 @@ PAGE = 64          # tokens per cache page (MF_PAGE in csrc/common.h)
 HAVE_PREFILL_ATTENTION = True
 PREFILL_MAX_SHARES = 8  # workgroups that may take the pages of one block of queries of the prompt attention in turn
 PREFILL_MIN_PAGES = 4   # ... each with at least this many pages
-EPI_F32, EPI_ACC_F32, EPI_BF16, EPI_SWIGLU = 0, 1, 2, 3
+EPI_F32, EPI_ACC_F32, EPI_BF16, EPI_SWIGLU, EPI_XIELU = 0, 1, 2, 3, 4
 
 
 class KernelError(RuntimeError):
@@ -824,7 +824,8 @@ def _need_tiled(tiled: Optional[torch.Tensor], name: str, n: int, k: int) -> Non
 
 
 def linear(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor], out: torch.Tensor,
-           accumulate: bool = False, variant: int = 0, tiled: Optional[torch.Tensor] = None) -> None:
+           accumulate: bool = False, variant: int = 0, tiled: Optional[torch.Tensor] = None,
+           xielu: bool = False) -> None:
     """out (+)= x @ weight^T (+ bias).  weight is [out][in].  float32 weights take the true
     32-bit kernel; bfloat16 weights take the matrix-core kernels (a few rows: the streaming
     kernel).  `out` is float32, or bfloat16 for a bfloat16 product that is stored.  `tiled`:
@@ -836,7 +837,11 @@ def linear(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor], 
     if weight.shape[1] != k:
         raise KernelError(f"linear: x is [{m},{k}], weight is {tuple(weight.shape)}")
     _need(out, "linear.out", _FLOATS, (m, n))
-    if bias is not None:
+    if xielu:
+        if bias is None or x.dtype != torch.bfloat16 or out.dtype != torch.bfloat16 or accumulate:
+            raise KernelError("linear(xielu): needs bfloat16 operands and output, and the biases with the two constants")
+        _need(bias, "linear.bias", torch.float32, (n + 2,))
+    elif bias is not None:
         _need(bias, "linear.bias", torch.float32, (n,))
     if m == 0:
         return
@@ -847,7 +852,7 @@ def linear(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor], 
         return
     if accumulate and out.dtype != torch.float32:
         raise KernelError("linear: accumulation needs a float32 output")
-    epi = EPI_BF16 if out.dtype == torch.bfloat16 else (EPI_ACC_F32 if accumulate else EPI_F32)
+    epi = EPI_XIELU if xielu else (EPI_BF16 if out.dtype == torch.bfloat16 else (EPI_ACC_F32 if accumulate else EPI_F32))
     aligned = not (x.data_ptr() % 16 or weight.data_ptr() % 16 or k % 8)
     if m <= 64 and variant == 0:
         splits, per = _k_split(m, n, k, False, aligned, tiled=tiled is not None)

@@ -104,12 +104,20 @@ class DenseXIELU(FeedForward):
         self.down = Linear(get(n["down"]), get(n["down"] + ".b"))
         pq = [float(v) for v in get(n["act"]).to(torch.float32).cpu()]
         self.a_pos, self.a_neg = _softplus(pq[0]), 0.5 + _softplus(pq[1])
+        # bfloat16 products apply the activation in their epilogue: its constants ride behind the biases
+        self.up_act_bias = None
+        if self.rt.is_bf16 and self.up.weight.dtype == torch.bfloat16:
+            tail = torch.tensor([self.a_pos, self.a_neg], dtype=torch.float32, device=self.up.bias.device)
+            self.up_act_bias = torch.cat([self.up.bias, tail]).contiguous()
 
     def decode_copies(self, make: bool, min_row_length: int = 0) -> int:
         return self.up.decode_copy(make, min_row_length) + self.down.decode_copy(make, min_row_length)
 
     def forward(self, x, h, ctx, accumulate: bool = True) -> None:
-        u = self.up(x, out_dtype=torch.float32)
         y = torch.empty((x.shape[0], self.inter), dtype=self.rt.dtype, device=x.device)
-        ops.xielu(u, y, self.a_pos, self.a_neg)
+        if self.up_act_bias is not None and x.dtype == torch.bfloat16:
+            ops.linear(x, self.up.weight, self.up_act_bias, y, tiled=self.up.tiled, xielu=True)
+        else:
+            u = self.up(x, out_dtype=torch.float32)
+            ops.xielu(u, y, self.a_pos, self.a_neg)
         self.down(y, out=h, accumulate=accumulate)

@@ -99,8 +99,16 @@ def rope_inplace(qkv, cos, sin, positions, n_rot_heads, n_heads_total, head_dim)
     x[:, :n_rot_heads] = torch.cat([v0 * c - v1 * s, v0 * s + v1 * c], dim=-1).float()
 
 
-def linear(x, weight, bias, out, accumulate=False, variant=0, tiled=None):
+def linear(x, weight, bias, out, accumulate=False, variant=0, tiled=None, xielu=False):
     y = x.double() @ weight.double().t()
+    if xielu:                            # the activation's constants ride behind the biases
+        n = weight.shape[0]
+        y = y + bias[:n].double()
+        a_pos, a_neg = float(bias[n]), float(bias[n + 1])
+        pos = a_pos * y * y + 0.5 * y
+        neg = a_neg * (torch.expm1(torch.clamp(y, max=0.0)) - y) + 0.5 * y
+        out.copy_(torch.where(y > 0, pos, neg).to(out.dtype))
+        return
     if bias is not None:
         y = y + bias.double()
     if accumulate:

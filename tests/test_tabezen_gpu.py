@@ -91,6 +91,19 @@ def test_xielu_kernel():
         assert err < (1e-6 if dtype == torch.float32 else 8e-3)
 
 
+@pytest.mark.parametrize("m, n, k", [(1, 112, 96), (8, 8192, 2048), (40, 200, 128), (300, 384, 256), (2048, 1000, 136)])
+def test_product_with_xielu_epilogue(m, n, k):
+    """Every size class of the bfloat16 product (few rows, split K, tiles) with the activation folded in."""
+    from minfer_amd.kernels import ops
+    x, w = rnd(m, k, seed=1).to(torch.bfloat16), rnd(n, k, seed=2, scale=k ** -0.5).to(torch.bfloat16)
+    bias = torch.cat([rnd(n, seed=3, scale=0.5), torch.tensor([0.8, 1.3])])
+    want, got = torch.empty(m, n, dtype=torch.bfloat16), torch.empty(m, n, dtype=torch.bfloat16, device=DEV)
+    plain_ops.linear(x, w, bias, want, xielu=True)
+    ops.linear(x.to(DEV), w.to(DEV), bias.to(DEV), got, xielu=True)
+    err = ((got.cpu().float() - want.float()).abs() / (1 + want.float().abs())).max()
+    assert err < 1e-2
+
+
 def test_pair_rotation_tables_and_kernel():
     from minfer_amd.kernels import ops
     from minfer_amd.parts.rotary import blended_frequencies
