@@ -224,6 +224,72 @@ __global__ __launch_bounds__(256) void headwise_mfma_kernel(const bf16* __restri
   }
 }
 
+// Prompts: a head's whole matrix (NO x NI, at most 150 KB with its padding) is staged in LDS once by
+// a workgroup of 8 waves, which then takes 128 tokens: a wave holds its 16 tokens' inputs in
+// registers (NI <= 512) and walks the outputs 16 at a time with the matrix's fragments from LDS
+// (rows 16 bytes apart in the banks).  The matrix is read from memory once per 128 tokens
+// instead of once per 16.
+#define MF_HW_KS_MAX 16
+__global__ __launch_bounds__(512) void headwise_lds_kernel(const bf16* __restrict__ in, int in_stride,
+                                                           const bf16* __restrict__ wo, bf16* __restrict__ out,
+                                                           int out_stride, const float* __restrict__ gate, int n_tok,
+                                                           int H, int NI, int NO) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char hw_smem[];
+  bf16* Ws = reinterpret_cast<bf16*>(hw_smem);
+  const int WSTR = NI + 8;
+  const int h = blockIdx.y;
+  const int chunks = NI / 8;
+  const int NO16 = (NO + 15) / 16 * 16;
+  for (int idx = threadIdx.x; idx < NO16 * chunks; idx += 512) {
+    const int o = idx / chunks, c = idx % chunks;
+    hw_u32x4 v = {0u, 0u, 0u, 0u};
+    if (o < NO) v = *reinterpret_cast<const hw_u32x4*>(wo + ((size_t)h * NO + o) * NI + c * 8);
+    *reinterpret_cast<hw_u32x4*>(Ws + (size_t)o * WSTR + c * 8) = v;
+  }
+  __syncthreads();
+  const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+  const int r16 = lane & 15, q4 = lane >> 4;
+  const int t = blockIdx.x * 128 + wv * 16 + r16;
+  const bool tok_ok = t < n_tok;
+  const bf16* xrow = in + ((size_t)(tok_ok ? t : 0) * H + h) * in_stride;
+  const int nks = (NI + 31) / 32;
+  hw_u32x4 xb[MF_HW_KS_MAX];
+#pragma unroll
+  for (int ks = 0; ks < MF_HW_KS_MAX; ++ks) {
+    const int i = 32 * ks + 8 * q4;
+    xb[ks] = hw_u32x4{0u, 0u, 0u, 0u};
+    if (ks < nks && tok_ok && i < NI) xb[ks] = *reinterpret_cast<const hw_u32x4*>(xrow + i);
+  }
+  if (blockIdx.x * 128 + wv * 16 >= n_tok) return;      // (after the barrier; uniform over the wave)
+  const float g = (gate && tok_ok) ? gate[(size_t)t * H + h] : 1.0f;
+  bf16* orow = out + ((size_t)(tok_ok ? t : 0) * H + h) * out_stride;
+  for (int mt = 0; mt < NO16 / 16; ++mt) {
+    floatx4 acc = {0.f, 0.f, 0.f, 0.f};
+    const bf16* wrow = Ws + (size_t)(mt * 16 + r16) * WSTR + 8 * q4;
+#pragma unroll
+    for (int ks = 0; ks < MF_HW_KS_MAX; ++ks) {
+      if (ks < nks) {
+        hw_u32x4 wa = {0u, 0u, 0u, 0u};
+        if (32 * ks + 8 * q4 < NI) wa = *reinterpret_cast<const hw_u32x4*>(wrow + 32 * ks);
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, wa), __builtin_bit_cast(bf16x8, xb[ks]),
+                                                      acc, 0, 0, 0);
+      }
+    }
+    if (!tok_ok) continue;
+    const int o0 = mt * 16 + 4 * q4;
+    if (o0 + 3 < NO && (out_stride & 3) == 0) {
+      bf16x4 v;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) v[i] = (bf16)(acc[i] * g);
+      *reinterpret_cast<bf16x4*>(orow + o0) = v;
+    } else {
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        if (o0 + i < NO) orow[o0 + i] = (bf16)(acc[i] * g);
+    }
+  }
+}
+
 MF_API int mf_headwise_mfma(const void* in, int in_stride, const void* wo, void* out, int out_stride,
                             const float* gate, int n_tok, int H, int NI, int NO, hipStream_t stream) {
   if (n_tok <= 0) return 0;
@@ -231,6 +297,19 @@ MF_API int mf_headwise_mfma(const void* in, int in_stride, const void* wo, void*
       (uintptr_t)out % 8)
     return (int)hipErrorInvalidValue;
   const int n_ttiles = (n_tok + 15) / 16;
+  const size_t lds = (size_t)((NO + 15) / 16 * 16) * (NI + 8) * 2;
+  if (n_tok >= 256 && NI <= 32 * MF_HW_KS_MAX && lds <= 150 * 1024) {
+    static bool raised = false;
+    if (!raised) {
+      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(headwise_lds_kernel),
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, 150 * 1024);
+      if (e != hipSuccess) return (int)e;
+      raised = true;
+    }
+    headwise_lds_kernel<<<dim3((n_tok + 127) / 128, H), 512, lds, stream>>>(
+        (const bf16*)in, in_stride, (const bf16*)wo, (bf16*)out, out_stride, gate, n_tok, H, NI, NO);
+    return mf_launch_status();
+  }
   if (n_tok <= 16) {
     const int n_otiles = (NO + 15) / 16;
     const long long tasks = (long long)H * n_otiles * n_ttiles;

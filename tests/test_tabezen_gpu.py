@@ -162,7 +162,9 @@ def test_headwise_linear_kernel():
 
 
 @pytest.mark.parametrize("n_tok, heads, n_in, n_out, stride", [(11, 3, 40, 290, 48), (1, 16, 128, 512, 128),
-                                                              (100, 5, 72, 8, 72), (8, 2, 264, 40, 264)])
+                                                              (100, 5, 72, 8, 72), (8, 2, 264, 40, 264),
+                                                              (300, 3, 128, 500, 136), (1000, 2, 512, 120, 512),
+                                                              (257, 4, 40, 90, 48)])
 def test_headwise_linear_matrix_core_kernel(n_tok, heads, n_in, n_out, stride):
     from minfer_amd.kernels import ops
     x = rnd(n_tok, heads, stride, seed=8).to(torch.bfloat16)
