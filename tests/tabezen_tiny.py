@@ -79,3 +79,36 @@ def write_tabezen(folder: str, raw: dict, seed: int = 0, sharpen: float = 1.0) -
     write_safetensors(os.path.join(folder, "model.safetensors"),
                       [(n, tuple(t.shape), torch.bfloat16) for n, t in made.items()], lambda n: made[n])
     return folder
+
+
+def random_config(rng) -> dict:
+    """A configuration drawn at random: widths and vocabularies that are multiples of nothing useful,
+    one to five layers of either kind in any order, borrowed tensors, layers without feed-forward, odd
+    head sizes, ranks and value widths, fewer rotated values than the rotated part holds, plain and
+    stretched frequency ladders."""
+    width = int(rng.choice([48, 64, 100, 128, 136, 192, 256, 320]))
+    groups = int(rng.choice([g for g in (1, 2, 4, 5, 8, 3) if width % g == 0]))
+    layers = []
+    for _ in range(int(rng.integers(1, 6))):
+        if layers and rng.random() < 0.25:
+            j = int(rng.integers(0, len(layers)))
+            if "weights_of" not in layers[j]:
+                layers.append(dict(layers[j], weights_of=j))
+                continue
+        mlp = None if rng.random() < 0.2 else dict(kind="dense", ff=int(rng.choice([40, 64, 100, 256, 384, 777])))
+        if rng.random() < 0.45:
+            layers.append(dict(type="mingru", mixer=dict(width=int(rng.choice([24, 64, 100, 256, 384, 513]))), mlp=mlp))
+            continue
+        rot_dim = int(rng.choice([2, 4, 8, 16, 32, 64, 6]))
+        dims = int(rng.choice([d for d in (2, 4, 6, 8, 16, 32, 64) if d <= rot_dim]))
+        scaling = None
+        if rng.random() < 0.7:
+            scaling = dict(factor=float(rng.choice([2.0, 8.0, 32.0])), original=int(rng.choice([16, 128, 1024, 4096])),
+                           fast=float(rng.choice([8.0, 32.0])), slow=float(rng.choice([1.0, 2.0])))
+        layers.append(dict(type="latent_attention", mlp=mlp, mixer=latent(
+            int(rng.choice([1, 2, 3, 4, 6, 8, 16])), int(rng.choice([8, 16, 24, 32, 64, 5])), rot_dim,
+            int(rng.choice([8, 16, 32, 48, 64, 7])), int(rng.choice([16, 32, 64, 96, 128, 256, 30])),
+            float(rng.choice([0.05, 0.125, 0.3])), base=float(rng.choice([100.0, 10000.0, 500000.0])), dims=dims,
+            scaling=scaling)))
+    return dict(architecture="Tabezen", vocab=int(rng.choice([64, 300, 512, 1000])), width=width,
+                norm=dict(eps=float(rng.choice([1e-6, 1e-5])), groups=groups), layers=layers)

@@ -13,7 +13,7 @@ import torch
 import plain_ops
 import plain_tabezen as pt
 from replays import batch_steps, chunk_steps, requests_for, run_steps, tail_steps, whole_steps
-from tabezen_tiny import TZ, TZ_A, TZ_B, write_tabezen
+from tabezen_tiny import TZ, TZ_A, TZ_B, random_config, write_tabezen
 from tiny import random_tokens
 
 pytestmark = pytest.mark.gpu
@@ -348,6 +348,25 @@ def test_replays_agree_with_plain(folders, plains, name, dtype):
     compare(run_steps(eng, chunk_steps(reqs, [[r] for r in ids], sizes=(2,))), ref, dtype, f"{name} portions of 2", lo)
     compare(run_steps(eng, chunk_steps(reqs, [[r] for r in ids], sizes=(129, 3, 64))), ref, dtype, f"{name} portions of 129", lo)
     assert not eng.cache.live_slots()
+
+
+@pytest.mark.parametrize("seed", range(8))
+def test_configurations_drawn_at_random(tmp_path, seed):
+    """Whatever config.json may say: sizes, orders and options drawn at random, both run types,
+    whole, one by one, in batches and in portions."""
+    raw = random_config(np.random.default_rng(2000 + seed))
+    folder = write_tabezen(str(tmp_path / "m"), raw, seed=seed)
+    plain = pt.PlainTabezen.from_folder(folder)
+    reqs = requests_for(raw["vocab"], (1, 9, 70, 200, 131), seed=seed)
+    ref = {rid: plain.forward(toks) for rid, toks in reqs.items()}
+    ids = list(reqs)
+    for dtype in ("float32", "bfloat16"):
+        eng = engine_for(folder, dtype)
+        what = f"random configuration {seed} ({json.dumps(raw)[:300]})"
+        compare(run_steps(eng, whole_steps(reqs)), ref, dtype, what + " whole", SHARP)
+        compare(run_steps(eng, tail_steps(reqs, tail=33)), ref, dtype, what + " one by one", SHARP)
+        compare(run_steps(eng, batch_steps(reqs, [ids[:3], ids[3:]])), ref, dtype, what + " batches", SHARP)
+        compare(run_steps(eng, chunk_steps(reqs, [ids[:2], ids[2:]])), ref, dtype, what + " portions", SHARP)
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
