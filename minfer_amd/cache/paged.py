@@ -68,6 +68,19 @@ class StateRequest:
     dtype: torch.dtype = torch.float32
 
 
+def split_request(req):
+    """(KVRequest or None, StateRequest or None) of what a mixer asks for one entry: a request of
+    either kind, None, or a pair of both (attention that also carries a fixed-size state)."""
+    if req is None:
+        return None, None
+    parts = list(req) if isinstance(req, (tuple, list)) else [req]
+    kv = [r for r in parts if isinstance(r, KVRequest)]
+    st = [r for r in parts if isinstance(r, StateRequest)]
+    if len(kv) > 1 or len(st) > 1 or len(kv) + len(st) != len(parts):
+        raise CacheError(f"unknown cache request {req!r}: a KVRequest, a StateRequest, or one of each")
+    return (kv[0] if kv else None), (st[0] if st else None)
+
+
 class PagePool:
     """Free list of page ids with double-free and leak checks (host side only)."""
 
@@ -158,7 +171,7 @@ class KVGroup:
 
 
 class Cache:
-    """`requests[entry]` is a KVRequest, a StateRequest or None, one per cache entry of the
+    """`requests[entry]` is a KVRequest, a StateRequest, a pair of both or None, one per cache entry of the
     model's run order.  `max_tokens` is the most tokens all live sequences hold together,
     each rounded up to a multiple of 64; `max_seqs` bounds the live sequences.  `poison`
     (tests) fills pages with NaN when they are created and whenever they are given back."""
@@ -173,12 +186,14 @@ class Cache:
         by_request: Dict[KVRequest, List[int]] = {}
         self.state_requests: Dict[int, StateRequest] = {}
         for entry, req in sorted(requests.items()):
-            if isinstance(req, KVRequest):
-                by_request.setdefault(req, []).append(entry)
-            elif isinstance(req, StateRequest):
-                self.state_requests[entry] = req
-            elif req is not None:
-                raise CacheError(f"cache entry {entry}: unknown request {req!r}")
+            try:
+                kv, st = split_request(req)
+            except CacheError as e:
+                raise CacheError(f"cache entry {entry}: {e}") from None
+            if kv is not None:
+                by_request.setdefault(kv, []).append(entry)
+            if st is not None:
+                self.state_requests[entry] = st
         self.groups: List[KVGroup] = [KVGroup(r, es, self.n_pages, dtype, device, poison)
                                       for r, es in by_request.items()]
         self.group_of: Dict[int, KVGroup] = {e: g for g in self.groups for e in g.entries}

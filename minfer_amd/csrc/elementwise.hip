@@ -594,3 +594,91 @@ MF_API int mf_fill_normal(void* out, int is_bf16, size_t n, uint64_t seed, float
     fill_normal_kernel<float><<<blocks, 256, 0, stream>>>((float*)out, n, seed, std, round_bf16);
   return mf_launch_status();
 }
+
+// ---------------------------------------------------------------- table row + learned position row
+// out[r][:] = table[ids[r]][:] + pos_table[positions[r]][:], added in 32-bit.  An id or a position
+// outside its table gives a row of NaN, as `embed_kernel` does.
+template <typename TT>
+__global__ __launch_bounds__(256) void embed_pos_kernel(const TT* __restrict__ table, const TT* __restrict__ pos_table,
+                                                        const int* __restrict__ ids, const int* __restrict__ positions,
+                                                        float* __restrict__ out, int d, int vocab, int n_pos) {
+  const int row = blockIdx.x;
+  const int id = ids[row], p = positions[row];
+  float* o = out + (size_t)row * d;
+  if (id < 0 || id >= vocab || p < 0 || p >= n_pos) {
+    for (int i = threadIdx.x; i < d; i += 256) o[i] = __builtin_nanf("");
+    return;
+  }
+  const TT* src = table + (size_t)id * d;
+  const TT* ps = pos_table + (size_t)p * d;
+  for (int i = threadIdx.x; i < d; i += 256) o[i] = to_f32(src[i]) + to_f32(ps[i]);
+}
+
+MF_API int mf_embed_pos(const void* table, const void* pos_table, int tables_are_bf16, const int* ids,
+                        const int* positions, float* out, int rows, int d, int vocab, int n_pos, hipStream_t stream) {
+  if (rows <= 0) return 0;
+  if (tables_are_bf16)
+    embed_pos_kernel<bf16><<<rows, 256, 0, stream>>>((const bf16*)table, (const bf16*)pos_table, ids, positions, out, d,
+                                                      vocab, n_pos);
+  else
+    embed_pos_kernel<float><<<rows, 256, 0, stream>>>((const float*)table, (const float*)pos_table, ids, positions, out,
+                                                       d, vocab, n_pos);
+  return mf_launch_status();
+}
+
+// ---------------------------------------------------------------- gelu, tanh form
+// 0.5 z (1 + tanh(sqrt(2/pi) (z + 0.044715 z^3))), from 32-bit sums, rounded once.
+__device__ __forceinline__ float gelu_tanh_of(float z) {
+  return 0.5f * z * (1.0f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
+}
+template <typename OT>
+__global__ __launch_bounds__(256) void gelu_tanh_kernel(const float* __restrict__ x, OT* __restrict__ out, size_t n) {
+  const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (i < n) out[i] = from_f32<OT>(gelu_tanh_of(x[i]));
+}
+
+MF_API int mf_gelu_tanh(const float* x, void* out, int out_is_bf16, size_t n, hipStream_t stream) {
+  if (n == 0) return 0;
+  const unsigned blocks = (unsigned)((n + 255) / 256);
+  if (out_is_bf16)
+    gelu_tanh_kernel<bf16><<<blocks, 256, 0, stream>>>(x, (bf16*)out, n);
+  else
+    gelu_tanh_kernel<float><<<blocks, 256, 0, stream>>>(x, (float*)out, n);
+  return mf_launch_status();
+}
+
+// ---------------------------------------------------------------- weighted sum of row buffers
+// out[r][:] = sum_j w[j] x_j[row(j, r)][:], added in the order of j.  The first `n_indexed` buffers are
+// read at row row_idx[r] (they hold more rows than `out`), the others at row r.  Up to MF_WSUM_MAX
+// buffers a launch; the entry point chains launches for more (the later ones add onto `out`).
+#define MF_WSUM_MAX 32
+struct WsumPtrs { const float* p[MF_WSUM_MAX]; };
+__global__ __launch_bounds__(256) void weighted_sum_kernel(WsumPtrs src, int n, int n_indexed,
+                                                           const int* __restrict__ row_idx, const float* __restrict__ w,
+                                                           float* __restrict__ out, int d, int add) {
+  const int r = blockIdx.x;
+  const int ri = row_idx ? row_idx[r] : r;
+  float* o = out + (size_t)r * d;
+  for (int i = threadIdx.x; i < d; i += 256) {
+    float a = add ? o[i] : 0.f;
+    for (int j = 0; j < n; ++j) a = fmaf(w[j], src.p[j][(size_t)(j < n_indexed ? ri : r) * d + i], a);
+    o[i] = a;
+  }
+}
+
+// `ptrs`: host array of n device pointers
+MF_API int mf_weighted_sum(const void* const* ptrs, int n, int n_indexed, const int* row_idx, const float* w, float* out,
+                           int rows, int d, hipStream_t stream) {
+  if (rows <= 0 || d <= 0) return 0;
+  if (n <= 0 || !ptrs || !w || !out) return (int)hipErrorInvalidValue;
+  for (int j0 = 0; j0 < n; j0 += MF_WSUM_MAX) {
+    WsumPtrs a;
+    const int m = n - j0 < MF_WSUM_MAX ? n - j0 : MF_WSUM_MAX;
+    for (int j = 0; j < MF_WSUM_MAX; ++j) a.p[j] = j < m ? (const float*)ptrs[j0 + j] : nullptr;
+    const int idx = n_indexed - j0 < 0 ? 0 : (n_indexed - j0 > m ? m : n_indexed - j0);
+    weighted_sum_kernel<<<rows, 256, 0, stream>>>(a, m, idx, row_idx, w + j0, out, d, j0 > 0 ? 1 : 0);
+    const int rc = mf_launch_status();
+    if (rc) return rc;
+  }
+  return 0;
+}

@@ -39,17 +39,18 @@ RESERVE_FRACTION = 0.06
 
 def cache_bytes_per_token(requests: Dict[int, object], dtype: torch.dtype) -> int:
     """Bytes one token of one sequence takes in the cache: K and V of every entry."""
-    from ..cache.paged import KVRequest
+    from ..cache.paged import split_request
     elem = torch.empty((), dtype=dtype).element_size()
-    return sum(r.n_kv_heads * (r.head_dim + r.value_dim) * elem for r in requests.values() if isinstance(r, KVRequest))
+    kvs = [split_request(r)[0] for r in requests.values()]
+    return sum(r.n_kv_heads * (r.head_dim + r.value_dim) * elem for r in kvs if r is not None)
 
 
 def state_bytes_per_sequence(requests: Dict[int, object]) -> int:
     """Bytes of fixed-size state one sequence slot takes, over all entries that ask for state."""
-    from ..cache.paged import StateRequest
+    from ..cache.paged import split_request
     total = 0
-    for r in requests.values():
-        if isinstance(r, StateRequest):
+    for r in (split_request(q)[1] for q in requests.values()):
+        if r is not None:
             n = torch.empty((), dtype=r.dtype).element_size()
             for d in r.shape:
                 n *= int(d)

@@ -13,7 +13,7 @@ from typing import Callable, Dict
 import torch
 
 from ..kernels import ops, tuning
-from ..parts.base import (BLOCKS, EMBEDDINGS, FEED_FORWARDS, HEADS, MIXERS, NORMS, Runtime, make_part,
+from ..parts.base import (BLOCKS, COMBINERS, EMBEDDINGS, FEED_FORWARDS, HEADS, MIXERS, NORMS, Runtime, make_part,
                           normed_input)
 from ..parts.spec import BlockSpec, ModelSpec
 from ..weights.loader import TensorSpec
@@ -35,9 +35,14 @@ def _build_block(bs: BlockSpec, rt: Runtime):
     if missing or unknown:
         raise ValueError(f"{where}: norms missing {missing}, not known to the arrangement {unknown}; "
                          f"it takes {list(known)}")
-    return cls(None if bs.mixer is None else make_part(MIXERS, bs.mixer, rt, "mixer"),
-               None if bs.feed_forward is None else make_part(FEED_FORWARDS, bs.feed_forward, rt, "feed-forward"),
-               {name: make_part(NORMS, spec, rt, "norm") for name, spec in bs.norms.items()}, rt)
+    parts = (None if bs.mixer is None else make_part(MIXERS, bs.mixer, rt, "mixer"),
+             None if bs.feed_forward is None else make_part(FEED_FORWARDS, bs.feed_forward, rt, "feed-forward"),
+             {name: make_part(NORMS, spec, rt, "norm") for name, spec in bs.norms.items()}, rt)
+    if bs.combiner is None:
+        return cls(*parts)
+    if not cls.takes_combiner:
+        raise ValueError(f"{where}: this arrangement takes no combiner")
+    return cls(*parts, combiner=make_part(COMBINERS, bs.combiner, rt, "combiner"))
 
 
 class DecoderModel:

@@ -33,6 +33,9 @@ LIBRARIES: Dict[str, str] = {
     "attn_latent": "attn_latent.hip",
     "attn_latent_mfma": "attn_latent_mfma.hip",
     "recurrence": "recurrence.hip",
+    "linear_attention": "linear_attention.hip",
+    "attn_capped": "attn_capped.hip",
+    "moe": "moe.hip",
     "sampling": "sampling.hip",
     "probe": "probe.hip",
 }
@@ -41,7 +44,8 @@ DEFINES: Dict[str, List[str]] = {}
 HEADERS = {"host_random": ["random_normal.h"],
            "elementwise": ["common.h", "random_normal.h"],
            "attn_tokens_f32": ["common.h", "attn_tokens_impl.h"],
-           "attn_decode_bf16": ["common.h", "attn_tokens_impl.h", "noalloc.h"]}
+           "attn_decode_bf16": ["common.h", "attn_tokens_impl.h", "noalloc.h"],
+           "attn_capped": ["common.h", "attn_tokens_impl.h"]}
 
 HIPCC_FLAGS = ["-O3", "--offload-arch=gfx950", "-fPIC", "-shared", "-std=c++17",
                "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",

@@ -43,6 +43,27 @@ _PROTOTYPES = {
         "mf_xielu": [_P, _P, c_int, c_size_t, c_float, c_float, _P],
         "mf_rope_table_freqs": [_P, _P, _P, c_int, c_int, c_double, _P],
         "mf_rope_pairs_inplace": [_P, _P, _P, _P, c_int, c_int, c_int, c_int, c_int, _P],
+        "mf_embed_pos": [_P, _P, c_int, _P, _P, _P, c_int, c_int, c_int, c_int, _P],
+        "mf_gelu_tanh": [_P, _P, c_int, c_size_t, _P],
+        "mf_weighted_sum": [_P, c_int, c_int, _P, _P, _P, c_int, c_int, _P],
+    },
+    "linear_attention": {
+        "mf_la_chunk": [],
+        "mf_lightning_scan": [_P, _P, _P, _P, _P, _P, c_int, c_int, c_int, c_int, _P],
+        "mf_lightning_scan_chunked": [_P, _P, c_int, _P, _P, _P, _P, _P, _P, c_int, c_int, c_int, c_int, _P],
+        "mf_gated_rmsnorm": [_P, _P, c_int, _P, _P, c_int, c_int, c_int, c_float, _P],
+    },
+    "attn_capped": {
+        "mf_qkv_conv_prep": [_P, _P, c_int, _P, _P, _P, _P, _P, _P, _P, c_int, c_float, _P, _P, _P, c_int, _P, _P, _P,
+                             c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, _P],
+        "mf_capped_attn": [_P, _P, _P, _P, c_int, _P, _P, _P, _P, _P, c_int, c_int, c_int, c_int, c_int, c_int,
+                           c_float, c_float, c_int, c_int, c_int, _P],
+        "mf_rope_half_inplace": [_P, _P, _P, _P, c_int, c_int, c_int, c_int, c_int, _P],
+    },
+    "moe": {
+        "mf_moe_route": [_P, _P, _P, _P, c_int, c_int, c_int, c_int, c_int, _P],
+        "mf_moe_act": [_P, _P, _P, c_int, c_int, c_int, c_int, c_float, _P],
+        "mf_moe_sparse": [_P, _P, _P, _P, _P, _P, _P, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, _P],
     },
     "recurrence": {
         "mf_mingru_scan": [_P, _P, _P, _P, _P, c_int, c_int, c_int, _P],
@@ -496,6 +517,288 @@ def rope_pairs_inplace(qkv: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor, 
 
 
 # ------------------------------------------------------------------ recurrences
+
+# ------------------------------------------------------------------ table row plus position row, gelu, weighted sums
+def embed_pos(table: torch.Tensor, pos_table: torch.Tensor, ids: torch.Tensor, positions: torch.Tensor,
+              out: torch.Tensor) -> None:
+    """out[r] = table[ids[r]] + pos_table[positions[r]], added in 32-bit."""
+    _need(table, "embed_pos.table", _FLOATS)
+    _need(pos_table, "embed_pos.pos_table", table.dtype)
+    n, d = ids.numel(), table.shape[1]
+    if pos_table.dim() != 2 or pos_table.shape[1] != d:
+        raise KernelError(f"embed_pos: position table {tuple(pos_table.shape)} for rows of {d}")
+    _need(ids, "embed_pos.ids", torch.int32)
+    _need(positions, "embed_pos.positions", torch.int32, (n,))
+    _need(out, "embed_pos.out", torch.float32, (n, d))
+    _check(_fn("elementwise", "mf_embed_pos")(_ptr(table), _ptr(pos_table), _is_bf16(table), _ptr(ids), _ptr(positions),
+                                               _ptr(out), n, d, table.shape[0], pos_table.shape[0], _stream()), "embed_pos")
+
+
+def gelu_tanh(x: torch.Tensor, out: torch.Tensor) -> None:
+    """out = 0.5 x (1 + tanh(sqrt(2/pi) (x + 0.044715 x^3))) from 32-bit values, rounded once."""
+    _need(x, "gelu_tanh.x", torch.float32)
+    _need(out, "gelu_tanh.out", _FLOATS, tuple(x.shape))
+    _check(_fn("elementwise", "mf_gelu_tanh")(_ptr(x), _ptr(out), _is_bf16(out), x.numel(), _stream()), "gelu_tanh")
+
+
+def weighted_sum(buffers, weights: torch.Tensor, out: torch.Tensor, row_idx: Optional[torch.Tensor] = None,
+                 n_indexed: int = 0) -> None:
+    """out[r] = sum_j weights[j] buffers[j][row(j, r)], added in the order of j in 32-bit.  The first
+    `n_indexed` buffers are read at row `row_idx[r]`, the others at row r."""
+    n = len(buffers)
+    rows, d = out.shape
+    _need(out, "weighted_sum.out", torch.float32)
+    _need(weights, "weighted_sum.weights", torch.float32, (n,))
+    if n_indexed:
+        _need(row_idx, "weighted_sum.row_idx", torch.int32, (rows,))
+    for j, b in enumerate(buffers):
+        _need(b, f"weighted_sum.buffers[{j}]", torch.float32)
+        if b.shape[1] != d or (j >= n_indexed and b.shape[0] != rows):
+            raise KernelError(f"weighted_sum: buffer {j} is {tuple(b.shape)}, out is {tuple(out.shape)}")
+        if b.data_ptr() == out.data_ptr():
+            raise KernelError("weighted_sum: the output is one of the inputs")
+    ptrs = (c_void_p * n)(*[b.data_ptr() for b in buffers])
+    _check(_fn("elementwise", "mf_weighted_sum")(ptrs, n, int(n_indexed), _ptr(row_idx if n_indexed else None),
+                                                  _ptr(weights), _ptr(out), rows, d, _stream()), "weighted_sum")
+
+
+# ------------------------------------------------------------------ linear attention with decay
+LA_CHUNK = 64            # tokens of a chunk of the chunked form (MF_LA_CHUNK in csrc/linear_attention.hip)
+LA_CHUNKED_MAX_DIM = 128  # key width up to which the chunked form's tiles fit into LDS
+
+
+def la_chunks(host_new):
+    """The chunk table of the chunked linear attention for a step whose sequences bring `host_new`
+    tokens: int32 `[2][n_chunks]` (first token, tokens) followed by `[n_seqs + 1]` first chunks."""
+    t0s, ns, firsts = [], [], [0]
+    t = 0
+    for n in host_new:
+        for c0 in range(0, n, LA_CHUNK):
+            t0s.append(t + c0)
+            ns.append(min(LA_CHUNK, n - c0))
+        firsts.append(len(t0s))
+        t += n
+    return torch.tensor(t0s + ns + firsts, dtype=torch.int32), len(t0s)
+
+
+def lightning_scan(proj: torch.Tensor, cu_seqlens: torch.Tensor, slot_ids: torch.Tensor, decays: torch.Tensor,
+                   state: torch.Tensor, out: torch.Tensor, n_heads: int, dim: int, v_dim: int,
+                   chunks=None) -> None:
+    """Linear attention with a decay per head over a ragged step.  `proj` float32
+    `[tokens][2 H dim + 2 H v_dim]`: q | k | v | gate pre-activations (the gate is not read here);
+    `state` float32 `[slots][H][dim][v_dim]`, read and left at each sequence's last token for the rows
+    `slot_ids`; `out` float32 `[tokens][H v_dim]`.  With `chunks` (`la_chunks`, the table on the device
+    and its number of chunks) the sequences are walked in chunks side by side."""
+    n_tok = proj.shape[0]
+    n_seqs = slot_ids.numel()
+    _need(proj, "lightning_scan.proj", torch.float32, (n_tok, 2 * n_heads * (dim + v_dim)))
+    _need(cu_seqlens, "lightning_scan.cu_seqlens", torch.int32, (n_seqs + 1,))
+    _need(slot_ids, "lightning_scan.slot_ids", torch.int32, (n_seqs,))
+    _need(decays, "lightning_scan.decays", torch.float32, (n_heads,))
+    _need(state, "lightning_scan.state", torch.float32)
+    if tuple(state.shape[1:]) != (n_heads, dim, v_dim):
+        raise KernelError(f"lightning_scan: state {tuple(state.shape)} for {n_heads} heads of {dim} x {v_dim}")
+    _need(out, "lightning_scan.out", torch.float32, (n_tok, n_heads * v_dim))
+    if dim > 256:
+        raise KernelError(f"lightning_scan: key width {dim} is beyond 256")
+    if chunks is None or dim > LA_CHUNKED_MAX_DIM:
+        _check(_fn("linear_attention", "mf_lightning_scan")(_ptr(proj), _ptr(cu_seqlens), _ptr(slot_ids), _ptr(decays),
+                                                            _ptr(state), _ptr(out), n_seqs, n_heads, dim, v_dim,
+                                                            _stream()), "lightning_scan")
+        return
+    table, n_chunks = chunks
+    _need(table, "lightning_scan.chunks", torch.int32, (2 * n_chunks + n_seqs + 1,))
+    ws = workspace("la_chunks", n_chunks * n_heads * dim * v_dim, proj.device)
+    first = c_void_p(table.data_ptr() + 8 * n_chunks)
+    _check(_fn("linear_attention", "mf_lightning_scan_chunked")(
+        _ptr(proj), _ptr(table), n_chunks, first, _ptr(slot_ids), _ptr(decays), _ptr(state), _ptr(ws), _ptr(out),
+        n_seqs, n_heads, dim, v_dim, _stream()), "lightning_scan_chunked")
+
+
+def gated_rmsnorm(o: torch.Tensor, proj: torch.Tensor, gate_offset: int, weight: torch.Tensor, eps: float,
+                  out: torch.Tensor) -> None:
+    """out = o / sqrt(mean(o^2) + eps) * weight * sigmoid(gate), the gate being the columns
+    `gate_offset ..` of the 32-bit rows `proj`."""
+    rows, n = o.shape
+    _need(o, "gated_rmsnorm.o", torch.float32)
+    _need(proj, "gated_rmsnorm.proj", torch.float32)
+    if proj.shape[0] != rows or gate_offset + n > proj.shape[1]:
+        raise KernelError(f"gated_rmsnorm: gate columns {gate_offset}..{gate_offset + n} of rows {tuple(proj.shape)}")
+    _need(weight, "gated_rmsnorm.weight", torch.float32, (n,))
+    _need(out, "gated_rmsnorm.out", _FLOATS, (rows, n))
+    _check(_fn("linear_attention", "mf_gated_rmsnorm")(_ptr(o), c_void_p(proj.data_ptr() + 4 * gate_offset), proj.shape[1],
+                                                       _ptr(weight), _ptr(out), _is_bf16(out), rows, n, float(eps),
+                                                       _stream()), "gated_rmsnorm")
+
+
+# ------------------------------------------------------------------ capped attention with a convolution in front
+CONV_MAX_TAPS = 16
+
+
+def rope_half_inplace(rows: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor, positions: torch.Tensor,
+                      n_rot_heads: int, n_heads_total: int, head_dim: int) -> None:
+    """Half-split rotation over the first 2 x cos.shape[1] values of the first `n_rot_heads` heads of
+    32-bit rows `[tokens][n_heads_total head_dim]`, in place."""
+    n_tok = positions.numel()
+    rot = 2 * cos.shape[1]
+    _need(rows, "rope_half.rows", torch.float32, (n_tok, n_heads_total * head_dim))
+    _need(cos, "rope_half.cos", torch.float32)
+    _need(sin, "rope_half.sin", torch.float32, tuple(cos.shape))
+    _need(positions, "rope_half.positions", torch.int32)
+    if rot > head_dim:
+        raise KernelError(f"rope_half: {rot} rotated values in heads of {head_dim}")
+    _check(_fn("attn_capped", "mf_rope_half_inplace")(_ptr(rows), _ptr(cos), _ptr(sin), _ptr(positions), n_tok,
+                                                      n_rot_heads, n_heads_total, head_dim, rot, _stream()), "rope_half_inplace")
+
+
+def qkv_conv_prep(qkv: torch.Tensor, conv_w: Optional[torch.Tensor], conv_state: Optional[torch.Tensor],
+                  cu_seqlens: torch.Tensor, seq_of_tok: torch.Tensor, slot_ids: torch.Tensor, positions: torch.Tensor,
+                  cos: Optional[torch.Tensor], sin: Optional[torch.Tensor], blend: float,
+                  v_first: Optional[torch.Tensor], v_own: Optional[torch.Tensor], page_table: torch.Tensor,
+                  q_out: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tensor, n_heads: int, n_kv_heads: int,
+                  dim: int, v_dim: int, write_cache: bool = True) -> None:
+    """From the 32-bit q|k|v rows of one product: the short causal convolution over time on every
+    channel (`conv_w` `[channels][taps]`; the rows before a sequence's part of the step come from
+    `conv_state` `[slots][taps - 1][channels]`, which is moved on afterwards), the half-split rotation of
+    q and k over the tables' 2 x columns first values of a head, v <- (1 - blend) v + blend v_first
+    where `v_first` is given, the convolved v into `v_own` where given, k and v into the cache pages
+    at the tokens' positions and q rounded into `q_out`."""
+    n_tok = positions.numel()
+    n_seqs = slot_ids.numel()
+    C = n_heads * dim + n_kv_heads * (dim + v_dim)
+    _need(qkv, "qkv_conv_prep.qkv", torch.float32, (n_tok, C))
+    taps = 1
+    if conv_w is not None:
+        _need(conv_w, "qkv_conv_prep.conv_w", torch.float32)
+        if conv_w.dim() != 2 or conv_w.shape[0] != C or not 1 <= conv_w.shape[1] <= CONV_MAX_TAPS:
+            raise KernelError(f"qkv_conv_prep: convolution weights {tuple(conv_w.shape)} for {C} channels")
+        taps = conv_w.shape[1]
+    if taps > 1:
+        _need(conv_state, "qkv_conv_prep.conv_state", torch.float32)
+        if tuple(conv_state.shape[1:]) != (taps - 1, C):
+            raise KernelError(f"qkv_conv_prep: state {tuple(conv_state.shape)} for {taps} taps of {C} channels")
+    rot = 0
+    if cos is not None:
+        _need(cos, "qkv_conv_prep.cos", torch.float32)
+        _need(sin, "qkv_conv_prep.sin", torch.float32, tuple(cos.shape))
+        rot = 2 * cos.shape[1]
+        if rot > dim:
+            raise KernelError(f"qkv_conv_prep: {rot} rotated values in heads of {dim}")
+    for name, t in (("v_first", v_first), ("v_own", v_own)):
+        if t is not None:
+            _need(t, "qkv_conv_prep." + name, torch.float32, (n_tok, n_kv_heads * v_dim))
+    _need(q_out, "qkv_conv_prep.q_out", _FLOATS, (n_tok, n_heads * dim))
+    _need_kv_pages("qkv_conv_prep", kcache, vcache, q_out.dtype, n_kv_heads, dim, v_dim)
+    _need(page_table, "qkv_conv_prep.page_table", torch.int32)
+    for name, t, shape in (("cu_seqlens", cu_seqlens, (n_seqs + 1,)), ("seq_of_tok", seq_of_tok, (n_tok,)),
+                           ("slot_ids", slot_ids, (n_seqs,)), ("positions", positions, (n_tok,))):
+        _need(t, "qkv_conv_prep." + name, torch.int32, shape)
+    if C * 4 > 159 * 1024:
+        raise KernelError(f"qkv_conv_prep: rows of {C} channels do not fit into LDS")
+    _check(_fn("attn_capped", "mf_qkv_conv_prep")(
+        _ptr(qkv), _ptr(conv_w), taps, _ptr(conv_state if taps > 1 else None), _ptr(cu_seqlens), _ptr(seq_of_tok),
+        _ptr(slot_ids), _ptr(positions), _ptr(cos), _ptr(sin), rot, float(blend), _ptr(v_first), _ptr(v_own),
+        _ptr(page_table), page_table.shape[1], _ptr(q_out), _ptr(kcache), _ptr(vcache), _is_bf16(q_out), n_tok, n_seqs,
+        n_heads, n_kv_heads, dim, v_dim, 1 if write_cache else 0, _stream()), "qkv_conv_prep")
+
+
+def _need_kv_pages(what: str, kcache: torch.Tensor, vcache: torch.Tensor, dtype, n_kv_heads: int, dim: int,
+                   v_dim: int) -> None:
+    _need(kcache, what + ".kcache", dtype)
+    _need(vcache, what + ".vcache", dtype)
+    if tuple(kcache.shape[1:]) != (n_kv_heads, PAGE, dim):
+        raise KernelError(f"{what}.kcache: shape {tuple(kcache.shape)}, expected [pages, {n_kv_heads}, {PAGE}, {dim}]")
+    want = v_page_shape(n_kv_heads, v_dim, dtype)
+    if tuple(vcache.shape[1:]) != want or vcache.shape[0] != kcache.shape[0]:
+        raise KernelError(f"{what}.vcache: shape {tuple(vcache.shape)}, expected {[kcache.shape[0]] + list(want)}")
+
+
+def capped_attn(q: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tensor, page_table: torch.Tensor,
+                positions: torch.Tensor, seq_of_tok: torch.Tensor, temp: torch.Tensor, out: torch.Tensor,
+                n_heads: int, n_kv_heads: int, dim: int, v_dim: int, scale: float, cap: float, window: int,
+                max_len: int) -> None:
+    """Each query token attends to its sequence's cache rows lo..position with
+    s = cap tanh(q . k scale temp[head] / cap) (no cap where `cap` is 0), ordinary softmax; keys of
+    `dim` and values of `v_dim` values."""
+    n_tok = positions.numel()
+    _need(q, "capped_attn.q", _FLOATS, (n_tok, n_heads * dim))
+    _need(out, "capped_attn.out", q.dtype, (n_tok, n_heads * v_dim))
+    _need_kv_pages("capped_attn", kcache, vcache, q.dtype, n_kv_heads, dim, v_dim)
+    _need(page_table, "capped_attn.page_table", torch.int32)
+    _need(positions, "capped_attn.positions", torch.int32, (n_tok,))
+    _need(seq_of_tok, "capped_attn.seq_of_tok", torch.int32, (n_tok,))
+    _need(temp, "capped_attn.temp", torch.float32, (n_heads,))
+    if n_heads % n_kv_heads or dim > 512 or v_dim > 256:
+        raise KernelError(f"capped_attn: {n_heads} heads over {n_kv_heads}, keys of {dim} (at most 512), values of "
+                          f"{v_dim} (at most 256)")
+    if max_len > page_table.shape[1] * PAGE:
+        raise KernelError(f"capped_attn: max_len {max_len} exceeds the page table ({page_table.shape[1]} pages)")
+    reach = min(max_len, window) if window else max_len
+    n_splits, split_len = 1, max(PAGE, (max_len + PAGE - 1) // PAGE * PAGE)
+    if reach > 4 * PAGE and not (window and window < max_len):
+        n_splits, split_len = split_plan(n_tok, n_kv_heads, n_heads // n_kv_heads, 128, max_len)
+    part = workspace("attn", n_tok * n_heads * n_splits * (v_dim + 2), q.device) if n_splits > 1 else None
+    _check(_fn("attn_capped", "mf_capped_attn")(
+        _ptr(q), _ptr(kcache), _ptr(vcache), _ptr(page_table), page_table.shape[1], _ptr(positions), _ptr(seq_of_tok),
+        _ptr(temp), _ptr(out), _ptr(part), _is_bf16(q), n_tok, n_heads, n_kv_heads, dim, v_dim, float(scale),
+        float(cap or 0.0), int(window or 0), n_splits, split_len, _stream()), "capped_attn")
+
+
+# ------------------------------------------------------------------ mixture of experts
+MOE_MAX_EXPERTS = 1024
+
+
+def moe_route(logits: torch.Tensor, dense: torch.Tensor, chosen: torch.Tensor, weights: torch.Tensor,
+              n_groups: int, keep: int) -> None:
+    """From the router's 32-bit logits `[tokens][experts]`: softmax scores, the `keep` best of `n_groups`
+    groups of neighbouring experts (a group's score is its best expert's), the `chosen.shape[1]` best
+    experts of those groups, weighted by their scores over their sum.  `dense` `[tokens][experts]` gets the
+    weights at the chosen experts and 0 elsewhere; `chosen`, `weights` `[tokens][top]`."""
+    n_tok, E = logits.shape
+    top = chosen.shape[1]
+    _need(logits, "moe_route.logits", torch.float32)
+    _need(dense, "moe_route.dense", torch.float32, (n_tok, E))
+    _need(chosen, "moe_route.chosen", torch.int32, (n_tok, top))
+    _need(weights, "moe_route.weights", torch.float32, (n_tok, top))
+    if E > MOE_MAX_EXPERTS or E % n_groups or not 1 <= keep <= n_groups or not 1 <= top <= min(64, keep * (E // n_groups)):
+        raise KernelError(f"moe_route: {E} experts in {n_groups} groups, {keep} kept, {top} chosen")
+    _check(_fn("moe", "mf_moe_route")(_ptr(logits), _ptr(dense), _ptr(chosen), _ptr(weights), n_tok, E, n_groups, keep,
+                                       top, _stream()), "moe_route")
+
+
+def moe_act(gu: torch.Tensor, dense: torch.Tensor, out: torch.Tensor, limit: float) -> None:
+    """`gu` float32 `[tokens][experts][2 F]` (gate sums, then up sums): out `[tokens][experts F]` =
+    dense[t][e] g sigmoid(1.702 g) (u + 1) with g = min(gate, limit), u = clamp(up, -limit, limit)."""
+    n_tok, E = dense.shape
+    _need(dense, "moe_act.dense", torch.float32)
+    _need(gu, "moe_act.gu", torch.float32)
+    if gu.shape[0] != n_tok or gu.shape[1] % (2 * E):
+        raise KernelError(f"moe_act: rows {tuple(gu.shape)} for {E} experts")
+    F = gu.shape[1] // (2 * E)
+    _need(out, "moe_act.out", _FLOATS, (n_tok, E * F))
+    _check(_fn("moe", "mf_moe_act")(_ptr(gu), _ptr(dense), _ptr(out), _is_bf16(out), n_tok, E, F, float(limit),
+                                     _stream()), "moe_act")
+
+
+def moe_sparse(x: torch.Tensor, gate_up: torch.Tensor, down: torch.Tensor, chosen: torch.Tensor, weights: torch.Tensor,
+               out: torch.Tensor, n_experts: int, limit: float) -> None:
+    """The chosen experts only, for steps of few tokens: `gate_up` `[experts][2 F][K]` (an expert's gate
+    rows, then its up rows), `down` `[N][experts F]`; out `[tokens][N]` float32 += the weighted sum of the
+    chosen experts' outputs, choices added in their order."""
+    n_tok, K = x.shape
+    top = chosen.shape[1]
+    N, EF = down.shape
+    F = EF // n_experts
+    _need(x, "moe_sparse.x", _FLOATS)
+    _need(gate_up, "moe_sparse.gate_up", x.dtype, (2 * EF, K))
+    _need(down, "moe_sparse.down", x.dtype, (N, n_experts * F))
+    _need(chosen, "moe_sparse.chosen", torch.int32, (n_tok, top))
+    _need(weights, "moe_sparse.weights", torch.float32, (n_tok, top))
+    _need(out, "moe_sparse.out", torch.float32, (n_tok, N))
+    y = torch.empty((n_tok, top, F), dtype=x.dtype, device=x.device)
+    _check(_fn("moe", "mf_moe_sparse")(_ptr(x), _ptr(gate_up), _ptr(down), _ptr(chosen), _ptr(weights), _ptr(y), _ptr(out),
+                                        _is_bf16(x), n_tok, top, n_experts, F, K, N, float(limit), _stream()), "moe_sparse")
+
 SCAN_CHUNK = 32          # tokens of a chunk of the chunked scan (MF_SCAN_CHUNK in csrc/recurrence.hip)
 
 

@@ -206,6 +206,21 @@ class Head(Part):
     takes_normed = False
 
 
+class Combiner(Part):
+    """What goes on to the next block where that is not simply the block's result: a part that sees
+    every block's result as it is made (a learned sum over all results so far, for one).  A block
+    calls `enter` with the stream as it received it and runs its branches on the buffer `enter`
+    returns; it calls `leave` with its result (reduced to the rows `keep_rows` where the model
+    asked for that) and hands on what `leave` returns.  What a combiner keeps between blocks of one
+    step lives in the step's context."""
+
+    def enter(self, h: torch.Tensor, ctx) -> torch.Tensor:
+        return h
+
+    def leave(self, h: torch.Tensor, ctx, keep_rows=None) -> torch.Tensor:
+        raise NotImplementedError
+
+
 class Block:
     """An arrangement of parts: a mixer and a feed-forward (either may be None where the
     arrangement allows it) and norms under the names the arrangement gives them (`norm_names`;
@@ -217,11 +232,16 @@ class Block:
     needs_mixer = True
     needs_feed_forward = True
 
+    takes_combiner = False    # True: the arrangement calls its combiner's `enter` and `leave`
+
     def __init__(self, mixer: Optional[Mixer], feed_forward: Optional[FeedForward], norms: Dict[str, Norm],
-                 rt: Runtime):
+                 rt: Runtime, combiner: Optional[Combiner] = None):
         self.mixer, self.feed_forward = mixer, feed_forward
         self.norms = dict(norms)
         self.rt = rt
+        self.combiner = combiner
+        if combiner is not None and not self.takes_combiner:
+            raise ValueError(f"{type(self).__name__}: this arrangement takes no combiner")
 
     @property
     def mixer_norm(self) -> Optional[Norm]:
@@ -234,7 +254,7 @@ class Block:
     def parts(self):
         """Every part of the block that exists, norms in the order of `norm_names`."""
         named = [self.norms[n] for n in self.norm_names + self.optional_norms if n in self.norms]
-        return tuple(p for p in [self.mixer, self.feed_forward] + named if p is not None)
+        return tuple(p for p in [self.mixer, self.feed_forward] + named + [self.combiner] if p is not None)
 
     def first_norm(self) -> Optional[Norm]:
         """The norm that reads the residual stream first when this block runs, if it starts with
@@ -252,6 +272,7 @@ POSITIONS: Dict[str, type] = {}
 BLOCKS: Dict[str, type] = {}
 EMBEDDINGS: Dict[str, type] = {}
 HEADS: Dict[str, type] = {}
+COMBINERS: Dict[str, type] = {}
 
 
 def _registrar(table: Dict[str, type], what: str):
@@ -271,6 +292,7 @@ register_position = _registrar(POSITIONS, "position encoding")
 register_block = _registrar(BLOCKS, "block arrangement")
 register_embedding = _registrar(EMBEDDINGS, "embedding")
 register_head = _registrar(HEADS, "head")
+register_combiner = _registrar(COMBINERS, "combiner")
 
 
 def make_part(table: Dict[str, type], spec: PartSpec, rt: Runtime, what: str):

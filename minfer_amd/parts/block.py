@@ -118,3 +118,44 @@ class BranchNormBlock(Block):
             y = self._run(self.feed_forward, self._input(h, ctx), h.shape[0], h.shape[1], ctx)
             self._join(self.norms["feed_forward_out"], y, h, ctx, want_copy=keep_rows is None)
         return h
+
+
+@register_block("parallel")
+class ParallelBlock(Block):
+    """x + mixer(N1(x)) + feed_forward(N2(x)): both branches read the same x, each through a norm of
+    its own.  norms: "mixer" before the mixer, "feed_forward" before the feed-forward; a block without
+    a feed-forward has neither it nor its norm.  With a combiner, what goes on is what the combiner
+    makes of the block's result (`Combiner.enter` / `leave`).
+
+    The feed-forward's input is normed before the mixer adds into the stream; the mixer's own input
+    may stay lazy (its first product reads the stream before its last one writes)."""
+
+    needs_mixer = True
+    needs_feed_forward = False
+    norm_names = ("mixer",)
+    optional_norms = ("feed_forward",)
+    takes_combiner = True
+
+    def __init__(self, mixer, feed_forward, norms, rt, combiner=None):
+        super().__init__(mixer, feed_forward, norms, rt, combiner=combiner)
+        if (feed_forward is None) != ("feed_forward" not in self.norms):
+            raise ValueError("parallel block: the feed-forward and the norm before it come together or not at all")
+
+    def forward(self, h, ctx, entry: int, writes_cache: bool, keep_rows=None):
+        ctx.norm_next = ctx.norm_ahead = None
+        if self.combiner is not None:
+            h = self.combiner.enter(h, ctx)
+        x_ff = None
+        if self.feed_forward is not None:
+            x_ff = self.norms["feed_forward"].forward(h, row_idx=keep_rows)
+        x = normed_input(self.norms["mixer"], self.mixer, h)
+        self.mixer.forward(x, h, ctx, entry, writes_cache)
+        if keep_rows is not None:
+            kept = torch.empty((keep_rows.numel(), h.shape[1]), dtype=h.dtype, device=h.device)
+            ops.gather_rows(h, keep_rows, kept)
+            h = kept
+        if self.feed_forward is not None:
+            self.feed_forward.forward(x_ff, h, ctx)
+        if self.combiner is not None:
+            h = self.combiner.leave(h, ctx, keep_rows)
+        return h

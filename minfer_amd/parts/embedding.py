@@ -92,3 +92,24 @@ class LinearHead(Head):
 
     def forward(self, x, ctx=None) -> torch.Tensor:
         return self.linear(x, out_dtype=torch.float32)
+
+
+@register_embedding("token_position_embedding")
+class TokenPositionEmbedding(TokenEmbedding):
+    """The table's row plus a learned row for the token's position (not scaled), added in 32-bit.
+    params: name, positions (tensors), vocab_size, hidden_size, max_positions."""
+
+    def __init__(self, spec, rt):
+        super().__init__(spec, rt)
+        self.pos_name, self.max_positions = spec.params["positions"], int(spec.params["max_positions"])
+        self.pos = None
+
+    def tensor_specs(self):
+        return dict(super().tensor_specs(), **{self.pos_name: TensorSpec((self.max_positions, self.hidden))})
+
+    def load(self, get):
+        super().load(get)
+        self.pos = get(self.pos_name).to(self.weight.dtype).contiguous()
+
+    def forward(self, token_ids, out, ctx=None) -> None:
+        ops.embed_pos(self.weight, self.pos, token_ids, ctx.positions, out)

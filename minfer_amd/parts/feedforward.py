@@ -121,3 +121,35 @@ class DenseXIELU(FeedForward):
             u = self.up(x, out_dtype=torch.float32)
             ops.xielu(u, y, self.a_pos, self.a_neg)
         self.down(y, out=h, accumulate=accumulate)
+
+
+@register_feed_forward("dense_gelu")
+class DenseGelu(FeedForward):
+    """down(gelu(up x)) without biases, gelu in its tanh form, from the up product's 32-bit sums and
+    rounded once.  params: hidden_size, intermediate_size, up, down (tensor names)."""
+
+    takes_normed = True
+    can_overwrite = True
+
+    def __init__(self, spec, rt):
+        super().__init__(spec, rt)
+        p = spec.params
+        self.hidden, self.inter = int(p["hidden_size"]), int(p["intermediate_size"])
+        self.names = {k: p[k] for k in ("up", "down")}
+        self.up = self.down = None
+
+    def tensor_specs(self):
+        n = self.names
+        return {n["up"]: TensorSpec((self.inter, self.hidden)), n["down"]: TensorSpec((self.hidden, self.inter))}
+
+    def load(self, get):
+        self.up, self.down = Linear(get(self.names["up"])), Linear(get(self.names["down"]))
+
+    def decode_copies(self, make: bool, min_row_length: int = 0) -> int:
+        return self.up.decode_copy(make, min_row_length) + self.down.decode_copy(make, min_row_length)
+
+    def forward(self, x, h, ctx, accumulate: bool = True) -> None:
+        u = self.up(x, out_dtype=torch.float32)
+        y = torch.empty((u.shape[0], self.inter), dtype=self.rt.dtype, device=u.device)
+        ops.gelu_tanh(u, y)
+        self.down(y, out=h, accumulate=accumulate)

@@ -72,3 +72,17 @@ class GroupRMSNorm(Norm):
     def add_normed(self, y, h, cast_out: Optional[torch.Tensor] = None) -> None:
         """h += norm(y) in one kernel; `cast_out` (bfloat16) also gets the new rows rounded."""
         ops.group_rmsnorm(y, self.weight, self.eps, self.groups, h, add=True, cast_out=cast_out)
+
+
+@register_norm("scalar_rmsnorm")
+class ScalarRMSNorm(RMSNorm):
+    """RMS norm with one gain for the whole vector: x / sqrt(mean(x^2) + eps) * g, g a tensor of a single
+    number.  Kept as a vector of equal gains, so every kernel and fold of `rmsnorm` serves it.
+    params: size, eps, weight (tensor name)."""
+
+    def tensor_specs(self):
+        return {self.name: TensorSpec((), init="ones")}
+
+    def load(self, get):
+        g = get(self.name).to(torch.float32).reshape(1)
+        self.weight = g.expand(self.size).contiguous()

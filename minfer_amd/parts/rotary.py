@@ -119,3 +119,43 @@ class RotaryPairs(PositionEncoding):
         total = n_heads + 2 * n_kv_heads
         ops.rope_pairs_inplace(qkv, self.cos, self.sin, ctx.positions, n_heads + n_kv_heads, total,
                                qkv.shape[1] // total)
+
+
+@register_position("rope_half")
+class RotaryHalf(PositionEncoding):
+    """Half-split rotation over the first `dims` values of a head: value i < dims/2 turns with value
+    i + dims/2 by the angle position * f_i; what lies behind the first `dims` values passes unchanged.
+    The frequency ladder is `blended_frequencies` (plain without `scaling`).  params: dims, base, scaling
+    (None or dict(factor, original, fast, slow)), max_positions.  `half_tables` hands the tables
+    `[positions][dims / 2]` to a mixer that rotates inside its own kernels; `encode` is the plain form."""
+
+    def __init__(self, spec, rt):
+        super().__init__(spec, rt)
+        p = spec.params
+        self.dims, self.base = int(p["dims"]), float(p["base"])
+        self.scaling = p.get("scaling")
+        self.max_positions = int(p["max_positions"])
+        if self.dims % 2 or self.dims < 2:
+            raise ValueError(f"rope_half: {self.dims} rotated values do not form pairs")
+        self.freqs, self.magnitude = blended_frequencies(self.dims, self.base, self.scaling)
+        self.cos = self.sin = None
+
+    def prepare(self, max_len: int) -> None:
+        if max_len > self.max_positions:
+            raise ValueError(f"position {max_len - 1} is beyond the model's {self.max_positions} positions")
+        have = 0 if self.cos is None else self.cos.shape[0]
+        if max_len > have:
+            n = min(self.max_positions, max(FIRST_TABLE, 1 << (max_len - 1).bit_length()))
+            if self.cos is not None:
+                ops.note_replaced_buffer(self.cos)
+                ops.note_replaced_buffer(self.sin)
+            self.cos, self.sin = ops.rope_table_freqs(n, self.freqs, self.magnitude, self.rt.device)
+
+    def half_tables(self, max_len: int):
+        self.prepare(max_len)
+        return self.cos, self.sin
+
+    def encode(self, qkv, ctx, n_heads: int, n_kv_heads: int) -> None:
+        self.prepare(ctx.max_len)
+        total = n_heads + 2 * n_kv_heads
+        ops.rope_half_inplace(qkv, self.cos, self.sin, ctx.positions, n_heads + n_kv_heads, total, qkv.shape[1] // total)

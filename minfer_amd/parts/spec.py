@@ -41,6 +41,7 @@ class BlockSpec:
     mixer_norm: Optional[PartSpec] = None
     feed_forward_norm: Optional[PartSpec] = None
     norms: Mapping[str, PartSpec] = field(default_factory=dict)
+    combiner: Optional[PartSpec] = None       # what goes on to the next block, where not the block's result itself
 
     def __post_init__(self):
         norms = dict(self.norms)

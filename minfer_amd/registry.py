@@ -44,6 +44,8 @@ def _register_builtin() -> None:
     register_architecture(ARCHITECTURE, Qwen2Config)
     from .config import tabezen
     register_architecture(tabezen.ARCHITECTURE, tabezen.TabezenConfig)
+    from .config import lagedra
+    register_architecture(lagedra.ARCHITECTURE, lagedra.LagedraConfig)
 
 
 _register_builtin()

@@ -326,6 +326,199 @@ def latent_attn(q_abs, cache, page_table, positions, seq_of_tok, out, rank, scal
         out[i] = (torch.softmax(s, dim=-1) @ rows[:, :rank]).to(out.dtype)
 
 
+# ------------------------------------------------------------------ position rows, gelu, weighted sums
+def embed_pos(table, pos_table, ids, positions, out):
+    out.copy_((table[ids.long()].double() + pos_table[positions.long()].double()).to(torch.float32))
+
+
+def gelu_tanh(x, out):
+    z = x.double()
+    out.copy_((0.5 * z * (1.0 + torch.tanh(math.sqrt(2.0 / math.pi) * (z + 0.044715 * z ** 3)))).to(out.dtype))
+
+
+def weighted_sum(buffers, weights, out, row_idx=None, n_indexed=0):
+    acc = torch.zeros(out.shape, dtype=torch.float64)
+    for j, b in enumerate(buffers):
+        rows = b[row_idx.long()] if j < n_indexed else b
+        acc += float(weights[j]) * rows.double()
+    out.copy_(acc.to(torch.float32))
+
+
+# ------------------------------------------------------------------ linear attention with decay
+LA_CHUNK = 64
+LA_CHUNKED_MAX_DIM = 128
+
+
+def lightning_scan(proj, cu_seqlens, slot_ids, decays, state, out, n_heads, dim, v_dim, chunks=None):
+    H, D, V = n_heads, dim, v_dim
+    p = proj.double()
+    silu = lambda z: z * torch.sigmoid(z)
+    t_all = p.shape[0]
+    q = silu(p[:, :H * D]).view(t_all, H, D)
+    k = silu(p[:, H * D:2 * H * D]).view(t_all, H, D)
+    v = silu(p[:, 2 * H * D:2 * H * D + H * V]).view(t_all, H, V)
+    for b in range(slot_ids.numel()):
+        slot = int(slot_ids[b])
+        S = state[slot].double()
+        for t in range(int(cu_seqlens[b]), int(cu_seqlens[b + 1])):
+            S = decays.double()[:, None, None] * S + k[t][:, :, None] * v[t][:, None, :]
+            S = S.float().double()                       # the state is carried in 32-bit
+            out[t] = torch.einsum("hdv,hd->hv", S, q[t]).reshape(-1).float()
+        state[slot] = S.float()
+
+
+def gated_rmsnorm(o, proj, gate_offset, weight, eps, out):
+    x = o.double()
+    n = x.shape[1]
+    g = proj[:, gate_offset:gate_offset + n].double()
+    y = x / torch.sqrt((x * x).mean(dim=-1, keepdim=True) + eps) * weight.double() * torch.sigmoid(g)
+    out.copy_(y.to(out.dtype))
+
+
+# ------------------------------------------------------------------ capped attention with a convolution in front
+CONV_MAX_TAPS = 16
+
+
+def _rotate_half(v, c, s):
+    half = c.shape[-1]
+    a, b = v[..., :half], v[..., half:2 * half]
+    return torch.cat([a * c - b * s, b * c + a * s, v[..., 2 * half:]], dim=-1)
+
+
+def rope_half_inplace(rows, cos, sin, positions, n_rot_heads, n_heads_total, head_dim):
+    t = positions.numel()
+    x = rows.double().view(t, n_heads_total, head_dim).clone()
+    c, s = cos[positions.long()].double()[:, None, :], sin[positions.long()].double()[:, None, :]
+    x[:, :n_rot_heads] = _rotate_half(x[:, :n_rot_heads], c, s)
+    rows.copy_(x.view(t, -1).to(rows.dtype))
+
+
+def _store_v(vcache, page, in_page, g, row):
+    """One value row of kv head g into a page of either layout."""
+    if vcache.dtype == torch.bfloat16:               # [pages][kv][2][V][32]
+        vcache[page, g, in_page // 32, :, in_page % 32] = row.to(vcache.dtype)
+    else:
+        vcache[page, g, in_page] = row.to(vcache.dtype)
+
+
+def _load_v(vcache, pages, in_page, g):
+    if vcache.dtype == torch.bfloat16:
+        return vcache[pages, g, in_page // 32, :, in_page % 32].double()
+    return vcache[pages, g, in_page].double()
+
+
+def qkv_conv_prep(qkv, conv_w, conv_state, cu_seqlens, seq_of_tok, slot_ids, positions, cos, sin, blend, v_first, v_own,
+                  page_table, q_out, kcache, vcache, n_heads, n_kv_heads, dim, v_dim, write_cache=True):
+    t_all, C = qkv.shape
+    u = qkv.double()
+    y = u.clone()
+    taps = 1 if conv_w is None else conv_w.shape[1]
+    if taps > 1:
+        w = conv_w.double()
+        for b in range(slot_ids.numel()):
+            r0, r1 = int(cu_seqlens[b]), int(cu_seqlens[b + 1])
+            slot = int(slot_ids[b])
+            full = torch.cat([conv_state[slot].double(), u[r0:r1]], dim=0)
+            acc = torch.zeros((r1 - r0, C), dtype=torch.float64)
+            for j in range(taps):
+                acc += w[:, j] * full[j:j + (r1 - r0)]
+            y[r0:r1] = acc
+            if write_cache:
+                conv_state[slot] = full[full.shape[0] - (taps - 1):].float()
+    nq, nk = n_heads * dim, n_kv_heads * dim
+    q = y[:, :nq].view(t_all, n_heads, dim)
+    k = y[:, nq:nq + nk].view(t_all, n_kv_heads, dim)
+    v = y[:, nq + nk:].view(t_all, n_kv_heads, v_dim)
+    if cos is not None:
+        c, s = cos[positions.long()].double()[:, None, :], sin[positions.long()].double()[:, None, :]
+        q, k = _rotate_half(q, c, s), _rotate_half(k, c, s)
+    if v_own is not None:
+        v_own.copy_(v.reshape(t_all, -1).float())
+    if v_first is not None:
+        v = (1.0 - blend) * v + blend * v_first.double().view(t_all, n_kv_heads, v_dim)
+    q_out.copy_(q.reshape(t_all, nq).to(q_out.dtype))
+    if not write_cache:
+        return
+    for i in range(t_all):
+        pos = int(positions[i])
+        page = int(page_table[int(seq_of_tok[i]), pos // PAGE])
+        assert page >= 0
+        kcache[page, :, pos % PAGE] = k[i].to(kcache.dtype)
+        for g in range(n_kv_heads):
+            _store_v(vcache, page, pos % PAGE, g, v[i, g])
+
+
+def capped_attn(q, kcache, vcache, page_table, positions, seq_of_tok, temp, out, n_heads, n_kv_heads, dim, v_dim,
+                scale, cap, window, max_len):
+    t_all = positions.numel()
+    group = n_heads // n_kv_heads
+    qq = q.double().view(t_all, n_heads, dim)
+    for i in range(t_all):
+        p = int(positions[i])
+        lo = max(0, p - window + 1) if window else 0
+        pos = torch.arange(lo, p + 1)
+        pages = page_table[int(seq_of_tok[i])].long()[pos // PAGE]
+        assert (pages >= 0).all(), "attention reads a page that was given back"
+        for h in range(n_heads):
+            g = h // group
+            keys = kcache[pages, g, pos % PAGE].double()
+            vals = torch.stack([_load_v(vcache, int(pg), int(ip), g) for pg, ip in zip(pages, pos % PAGE)])
+            s = (keys @ qq[i, h]) * scale * float(temp[h])
+            if cap:
+                s = cap * torch.tanh(s / cap)
+            out[i, h * v_dim:(h + 1) * v_dim] = (torch.softmax(s, dim=0) @ vals).to(out.dtype)
+
+
+# ------------------------------------------------------------------ mixture of experts
+MOE_MAX_EXPERTS = 1024
+
+
+def moe_route(logits, dense, chosen, weights, n_groups, keep):
+    n_tok, E = logits.shape
+    top = chosen.shape[1]
+    per = E // n_groups
+    s = torch.softmax(logits.float(), dim=-1)
+    dense.zero_()
+    for t in range(n_tok):
+        gs = s[t].view(n_groups, per).max(dim=1).values
+        kept = torch.argsort(-gs, stable=True)[:keep]
+        masked = torch.full((E,), -1.0)
+        for g in kept.tolist():
+            masked[g * per:(g + 1) * per] = s[t, g * per:(g + 1) * per]
+        pick = torch.argsort(-masked, stable=True)[:top]
+        w = s[t, pick] / (s[t, pick].sum() + 1e-20)
+        chosen[t] = pick.to(torch.int32)
+        weights[t] = w
+        dense[t, pick] = w
+
+
+def _expert_act(g, u, limit):
+    g = torch.clamp(g, max=limit)
+    u = torch.clamp(u, -limit, limit)
+    return g * torch.sigmoid(1.702 * g) * (u + 1.0)
+
+
+def moe_act(gu, dense, out, limit):
+    n_tok, E = dense.shape
+    F = gu.shape[1] // (2 * E)
+    x = gu.double().view(n_tok, E, 2, F)
+    y = _expert_act(x[:, :, 0], x[:, :, 1], limit) * dense.double()[:, :, None]
+    out.copy_(y.reshape(n_tok, E * F).to(out.dtype))
+
+
+def moe_sparse(x, gate_up, down, chosen, weights, out, n_experts, limit):
+    n_tok, K = x.shape
+    N, EF = down.shape
+    F = EF // n_experts
+    gu = gate_up.double().view(n_experts, 2, F, K)
+    dn = down.double().view(N, n_experts, F)
+    for t in range(n_tok):
+        for k in range(chosen.shape[1]):
+            e = int(chosen[t, k])
+            y = _expert_act(gu[e, 0] @ x[t].double(), gu[e, 1] @ x[t].double(), limit).to(x.dtype).double()
+            out[t] += (float(weights[t, k]) * (dn[:, e] @ y)).float()
+
+
 # ------------------------------------------------------------------ sampling
 def argmax(logits, out):
     import plain_qwen2 as pq
@@ -397,7 +590,9 @@ NAMES = ["embed", "rmsnorm", "gather_rows", "swiglu", "convert", "fill_normal", 
          "rope_kvwrite", "rope_inplace", "linear", "attn_tokens", "attn_prefill", "argmax", "sample", "penalties",
          "top_k", "top_p", "sample_filtered", "sample_filtered_takes", "advance", "interleave_gate_up", "linear_swiglu", "linear_normed", "linear_fused", "attn_decode_rope",
          "group_rmsnorm", "xielu", "rope_table_freqs", "rope_pairs_inplace", "mingru_scan", "latent_prep",
-         "headwise_linear", "latent_attn", "headwise_mfma_takes", "headwise_linear_mfma"]
+         "headwise_linear", "latent_attn", "headwise_mfma_takes", "headwise_linear_mfma",
+         "embed_pos", "gelu_tanh", "weighted_sum", "lightning_scan", "gated_rmsnorm", "rope_half_inplace",
+         "qkv_conv_prep", "capped_attn", "moe_route", "moe_act", "moe_sparse"]
 
 
 def install(monkeypatch):
