@@ -178,7 +178,8 @@ class LagedraConfig:
                          schedule=straight_schedule(len(blocks)), max_positions=self.max_positions, stop_tokens=())
 
     def ignored_tensors(self) -> Tuple[str, ...]:
-        return ()
+        """A layer without a feed-forward has no use for the norm in front of one; a file may hold it."""
+        return tuple(f"l{i}.norm2" for i, layer in enumerate(self.layers) if layer["mlp"] is None)
 
     def random_init_std(self, tensor_name: str) -> float:
         """Standard deviation for random weights: `init_std` where the configuration gives one, else

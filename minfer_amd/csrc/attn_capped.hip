@@ -39,8 +39,8 @@ __global__ __launch_bounds__(256) void qkv_conv_prep_kernel(
   const int b = seq_of_tok[t];
   const int i = t - cu_seqlens[b];  // index of the token inside its sequence's part of the step
   const float* row = qkv + (size_t)t * C;
-  if (taps > 1) {
-    const float* st = conv_state + (size_t)slot_ids[b] * (taps - 1) * C;
+  if (conv_w) {
+    const float* st = taps > 1 ? conv_state + (size_t)slot_ids[b] * (taps - 1) * C : nullptr;
     for (int c = threadIdx.x; c < C; c += 256) {
       float a = 0.f;
       for (int j = 0; j < taps; ++j) {
@@ -283,7 +283,7 @@ MF_API int mf_qkv_conv_prep(const float* qkv, const float* conv_w, int taps, flo
                             int n_seqs, int H, int G, int D, int V, int write_cache, hipStream_t stream) {
   if (n_tok <= 0) return 0;
   const int C = H * D + G * D + G * V;
-  if (H <= 0 || G <= 0 || D <= 0 || V <= 0 || rot < 0 || rot % 2 || rot > D || taps > MF_CONV_MAX_TAPS ||
+  if (H <= 0 || G <= 0 || D <= 0 || V <= 0 || rot < 0 || rot % 2 || rot > D || taps < 1 || taps > MF_CONV_MAX_TAPS ||
       (taps > 1 && (!conv_w || !conv_state)) || (size_t)C * sizeof(float) > 160 * 1024 - 1024)
     return (int)hipErrorInvalidValue;
   const size_t lds = (size_t)C * sizeof(float);

@@ -555,8 +555,10 @@ def weighted_sum(buffers, weights: torch.Tensor, out: torch.Tensor, row_idx: Opt
         _need(b, f"weighted_sum.buffers[{j}]", torch.float32)
         if b.shape[1] != d or (j >= n_indexed and b.shape[0] != rows):
             raise KernelError(f"weighted_sum: buffer {j} is {tuple(b.shape)}, out is {tuple(out.shape)}")
-        if b.data_ptr() == out.data_ptr():
+        if rows and b.data_ptr() == out.data_ptr():
             raise KernelError("weighted_sum: the output is one of the inputs")
+    if rows == 0:
+        return
     ptrs = (c_void_p * n)(*[b.data_ptr() for b in buffers])
     _check(_fn("elementwise", "mf_weighted_sum")(ptrs, n, int(n_indexed), _ptr(row_idx if n_indexed else None),
                                                   _ptr(weights), _ptr(out), rows, d, _stream()), "weighted_sum")

@@ -24,7 +24,7 @@ from .linear import Linear
 @register_mixer("capped_attention")
 class CappedAttention(Mixer):
     """params: hidden_size, n_heads, n_kv_heads, dim, v_dim, scale, cap (None or 0: scores are not
-    capped), window (None or int), taps (None or 1: no convolution), position (PartSpec of a
+    capped), window (None or int), taps (None: no convolution), position (PartSpec of a
     half-split rotation with `half_tables`, or None), v_share (None, or the name under which the
     layers that blend their values find the first one's), v_share_first (True in the first of them),
     q, k, v, o, temp, vmix (tensor names; the convolutions are name + ".conv")."""
@@ -40,7 +40,8 @@ class CappedAttention(Mixer):
         self.scale = float(p["scale"])
         self.cap = float(p.get("cap") or 0.0)
         self.window = p.get("window")
-        self.taps = int(p.get("taps") or 1)
+        self.has_conv = p.get("taps") is not None
+        self.taps = int(p["taps"]) if self.has_conv else 1
         self.v_share, self.v_first = p.get("v_share"), bool(p.get("v_share_first", False))
         if self.nh % self.nk:
             raise ValueError(f"capped_attention: {self.nh} heads are not a multiple of {self.nk} kv heads")
@@ -64,7 +65,7 @@ class CappedAttention(Mixer):
         n = self.names
         rows = {"q": self.nh * self.dim, "k": self.nk * self.dim, "v": self.nk * self.vdim}
         s = {n[k]: TensorSpec((r, self.hidden)) for k, r in rows.items()}
-        if self.taps > 1:
+        if self.has_conv:
             s.update({n[k] + ".conv": TensorSpec((r, self.taps)) for k, r in rows.items()})
         s[n["o"]] = TensorSpec((self.hidden, self.nh * self.vdim))
         s[n["temp"]] = TensorSpec((self.nh,), init="ones")
@@ -76,7 +77,7 @@ class CappedAttention(Mixer):
         n = self.names
         self.qkv = Linear.stacked([get(n[k]) for k in ("q", "k", "v")])
         self.o = Linear(get(n["o"]))
-        if self.taps > 1:
+        if self.has_conv:
             self.conv = torch.cat([get(n[k] + ".conv").to(torch.float32) for k in ("q", "k", "v")], dim=0).contiguous()
         self.temp = get(n["temp"]).to(torch.float32).contiguous()
         if self.v_share is not None:
