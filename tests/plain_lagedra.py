@@ -184,7 +184,7 @@ def windowed_attention(h, w, m, v_first=None):
         k = rotate_half(k, pos, rot["dims"], rot["base"], rot.get("scaling"))
     own = v
     if v_first is not None:
-        lam = float(w["vmix"])
+        lam = float(np.asarray(w["vmix"]).reshape(()))
         v = (1.0 - lam) * v + lam * v_first
     window = (m.get("mask") or {}).get("size")
     cap = m.get("softcap")
@@ -227,7 +227,7 @@ class PlainLagedra:
         v_first = None
         for i, layer in enumerate(c["layers"]):
             p = f"l{i}."
-            a = scalar_rms_norm(x, float(w[p + "norm1"]), eps)
+            a = scalar_rms_norm(x, float(w[p + "norm1"].reshape(())), eps)
             m = layer["mixer"]
             if layer["type"] == "lightning":
                 y = lightning(a, self.sub(p + "mix."), m, eps)[0]
@@ -237,7 +237,7 @@ class PlainLagedra:
                 if mixes and v_first is None:
                     v_first = own
             if layer["mlp"] is not None:
-                b = scalar_rms_norm(x, float(w[p + "norm2"]), eps)
+                b = scalar_rms_norm(x, float(w[p + "norm2"].reshape(())), eps)
                 mw = self.sub(p + "mlp.")
                 y = y + (dense_ffn(b, mw["up"], mw["down"]) if layer["mlp"]["kind"] == "dense"
                          else moe_ffn(b, mw, layer["mlp"]))
@@ -245,7 +245,7 @@ class PlainLagedra:
             x = sum(w[p + "dwa"][j] * results[j] for j in range(i + 2))
             if layers_out is not None:
                 layers_out.append(x)
-        return scalar_rms_norm(x, float(w["final.norm"]), eps) @ w["head"].T
+        return scalar_rms_norm(x, float(w["final.norm"].reshape(())), eps) @ w["head"].T
 
 
 def greedy(logits_row) -> int:

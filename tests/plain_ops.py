@@ -413,17 +413,18 @@ def qkv_conv_prep(qkv, conv_w, conv_state, cu_seqlens, seq_of_tok, slot_ids, pos
     u = qkv.double()
     y = u.clone()
     taps = 1 if conv_w is None else conv_w.shape[1]
-    if taps > 1:
+    if conv_w is not None:
         w = conv_w.double()
         for b in range(slot_ids.numel()):
             r0, r1 = int(cu_seqlens[b]), int(cu_seqlens[b + 1])
             slot = int(slot_ids[b])
-            full = torch.cat([conv_state[slot].double(), u[r0:r1]], dim=0)
+            before = conv_state[slot].double() if taps > 1 else torch.zeros((0, C), dtype=torch.float64)
+            full = torch.cat([before, u[r0:r1]], dim=0)
             acc = torch.zeros((r1 - r0, C), dtype=torch.float64)
             for j in range(taps):
                 acc += w[:, j] * full[j:j + (r1 - r0)]
             y[r0:r1] = acc
-            if write_cache:
+            if write_cache and taps > 1:
                 conv_state[slot] = full[full.shape[0] - (taps - 1):].float()
     nq, nk = n_heads * dim, n_kv_heads * dim
     q = y[:, :nq].view(t_all, n_heads, dim)
