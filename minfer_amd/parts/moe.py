@@ -11,6 +11,9 @@ experts' matrices stacked), apply the activation times the token's weight for th
 was not chosen) and multiply by the experts' down matrices side by side: two products whatever
 the routing, experts / top times the arithmetic of the chosen experts alone.  Steps of few tokens
 read only the chosen experts' matrices (`ops.moe_sparse`).
+
+A step whose context carries a list under `_memo["route_log"]` gets every routed layer's choices
+(`[rows][top]` expert numbers, on the device) appended to it, in run order.
 """
 from __future__ import annotations
 
@@ -74,6 +77,9 @@ class GroupedMoE(FeedForward):
         chosen = torch.empty((n, self.top), dtype=torch.int32, device=dev)
         weights = torch.empty((n, self.top), dtype=torch.float32, device=dev)
         ops.moe_route(z, dense, chosen, weights, self.groups, self.keep)
+        log = ctx._memo.get("route_log") if ctx is not None else None
+        if log is not None:                  # a caller that wants to know: every routed layer's choices, in run order
+            log.append(chosen)
         if n <= SPARSE_UP_TO and x.dtype == self.gate_up.weight.dtype:
             if not accumulate:
                 h.zero_()

@@ -1,5 +1,5 @@
 """Small Lagedra configurations that differ in every size and option, a writer of model folders with
-random weights whose gains, sum weights, temperatures and blends are not the trivial ones, and
+random weights whose gains (0.6 to 1.4), sum weights, temperatures and blends are not the trivial ones, and
 configurations drawn at random."""
 from __future__ import annotations
 
@@ -96,7 +96,7 @@ def write_lagedra(folder: str, raw: dict, seed: int = 0, sharpen: float = 1.0) -
         elif name.endswith(".vmix"):
             a = rng.uniform(0.2, 0.6, shape)
         elif "norm" in name or name.endswith(".temp"):
-            a = 1.0 + 0.3 * rng.standard_normal(shape)
+            a = rng.uniform(0.6, 1.4, shape)
         elif name.endswith(".conv"):
             a = rng.standard_normal(shape) / np.sqrt(shape[1])
         elif name in ("embed", "pos"):

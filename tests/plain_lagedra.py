@@ -97,15 +97,47 @@ def route(z, top: int, n_groups: int, keep: int):
     return chosen, w
 
 
-def moe_ffn(h, w, m):
-    """h [t][width]; w: tensors of the feed-forward ("router", "e<i>.gate" ...); m: its config."""
+def route_margin(z, top: int, n_groups: int, keep: int) -> float:
+    """How far the router's decision for one token is from going the other way: the smallest gap, in
+    logits, between what was just taken and what was just left out (the last kept group against the
+    best group left out, the last chosen expert against the best one left out among the kept groups).
+    Infinite where nothing is left out.  A run in reduced precision may decide a token with a small
+    margin differently; a comparison passes such tokens over."""
+    per = len(z) // n_groups
+    gz = np.sort(z.reshape(n_groups, per).max(axis=1))[::-1]
+    margin = gz[keep - 1] - gz[keep] if keep < n_groups else math.inf
+    kept = np.argsort(-z.reshape(n_groups, per).max(axis=1), kind="stable")[:keep]
+    allowed = np.sort(np.concatenate([z[g * per:(g + 1) * per] for g in kept]))[::-1]
+    if top < len(allowed):
+        margin = min(margin, allowed[top - 1] - allowed[top])
+    return float(margin)
+
+
+def moe_ffn(h, w, m, margins=None, forced=None, choices=None):
+    """h [t][width]; w: tensors of the feed-forward ("router", "e<i>.gate" ...); m: its config.
+    `margins`, a list, gets every token's `route_margin`, `choices`, a list, the router's own choices
+    [t][top].  `forced` [t][top]: the experts to take instead
+    of the router's own choice (their weights are still their scores over the sum of their scores), for
+    a comparison with a run that decided a close call the other way."""
     r = m["router"]
     z = h @ w["router"].T
     out = np.zeros_like(h)
+    if margins is not None:
+        margins.append(np.array([route_margin(z[t], r["top"], r["groups"]["count"], r["groups"]["keep"])
+                                 for t in range(h.shape[0])]))
+    own = []
     for t in range(h.shape[0]):
         chosen, weights = route(z[t], r["top"], r["groups"]["count"], r["groups"]["keep"])
+        own.append(chosen)
+        if forced is not None:
+            chosen = np.asarray(forced[t])
+            sc = np.exp(z[t] - z[t].max())
+            sc = sc / sc.sum()
+            weights = sc[chosen] / (sc[chosen].sum() + 1e-20)
         for e, wt in zip(chosen, weights):
             out[t] += wt * expert(h[t], w[f"e{e}.gate"], w[f"e{e}.up"], w[f"e{e}.down"], m["expert"]["limit"])
+    if choices is not None:
+        choices.append(np.stack(own))
     return out
 
 
@@ -216,9 +248,11 @@ class PlainLagedra:
     def sub(self, prefix: str):
         return {n[len(prefix):]: t for n, t in self.w.items() if n.startswith(prefix)}
 
-    def forward(self, tokens, layers_out=None):
+    def forward(self, tokens, layers_out=None, margins=None, routes=None, choices=None):
         """Logits [t][vocab] of one sequence from position 0.  `layers_out`, a list, gets the stream
-        that leaves every layer."""
+        that leaves every layer; `margins`, a list, one array of `route_margin` per routed layer;
+        `routes`: layer number -> [t][top] experts to take in that layer, `choices`, a list, one array
+        [t][top] of the router's own choices per routed layer (`moe_ffn`)."""
         c, w = self.c, self.w
         eps = c["norm"]["eps"]
         T = len(tokens)
@@ -240,12 +274,16 @@ class PlainLagedra:
                 b = scalar_rms_norm(x, float(w[p + "norm2"].reshape(())), eps)
                 mw = self.sub(p + "mlp.")
                 y = y + (dense_ffn(b, mw["up"], mw["down"]) if layer["mlp"]["kind"] == "dense"
-                         else moe_ffn(b, mw, layer["mlp"]))
+                         else moe_ffn(b, mw, layer["mlp"], margins, None if routes is None else routes.get(i), choices))
             results.append(x + y)
             x = sum(w[p + "dwa"][j] * results[j] for j in range(i + 2))
             if layers_out is not None:
                 layers_out.append(x)
         return scalar_rms_norm(x, float(w["final.norm"].reshape(())), eps) @ w["head"].T
+
+
+    def routed_layers(self):
+        return [i for i, layer in enumerate(self.c["layers"]) if layer["mlp"] is not None and layer["mlp"]["kind"] == "moe"]
 
 
 def greedy(logits_row) -> int:

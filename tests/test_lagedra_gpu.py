@@ -24,25 +24,82 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 # deviation (measured 0.5 to 1.5 % rms at three and four layers); 32-bit in absolute terms
 BF16_RMS, BF16_MAX, F32_ABS = 0.04, 0.2, 2e-4
 SHARP = 3.0        # where the queries are scaled up so that single keys decide, the scores' roundings grow with them
+# A router decides a token between two experts (or groups) whose logits differ by less than this differently
+# in bfloat16 than in 64 bits now and then (seen at margins of 0.001 to 0.003); the token's row then differs
+# by a whole expert and the layers behind carry the difference on.  So a bfloat16 run is compared with the
+# plain implementation taking the run's own choices (`routes=`), and the choices themselves must be the
+# plain router's wherever its margin is at least this.  The 32-bit comparison forces nothing.
+CLOSE_CALL = 0.02
 
 
 def rnd(*shape, seed=0, scale=1.0):
     return torch.randn(*shape, generator=torch.Generator().manual_seed(seed)) * scale
 
 
-def compare(rows, ref, dtype, what, loosen=1.0, f32_abs=F32_ABS):
+def run_logged(engine, steps, routed_layers):
+    """`replays.run_steps` with the routed layers' choices: ({(request, position): logits row},
+    {request: {layer: [position] -> chosen experts}}).  Every step asks for all of its positions."""
+    slots, pos, rows, routes = {}, {}, {}, {}
+    for st in steps:
+        ents = st["entries"]
+        for e in ents:
+            assert e["want"] == list(range(len(e["tokens"])))
+            if e["id"] not in slots:
+                slots[e["id"]] = engine.new_sequence()
+                pos[e["id"]] = 0
+        ctx = engine.build_context([slots[e["id"]] for e in ents], [e["tokens"] for e in ents], [e["want"] for e in ents])
+        log = ctx._memo["route_log"] = []
+        logits = engine.model.forward(ctx).cpu().numpy()
+        engine.cache.commit(ctx.new_lengths)
+        assert len(log) == len(routed_layers)
+        chosen = [c.cpu().numpy() for c in log]
+        r = 0
+        for e in ents:
+            for w in e["want"]:
+                rows[(e["id"], pos[e["id"]] + w)] = logits[r]
+                for layer, c in zip(routed_layers, chosen):
+                    routes.setdefault(e["id"], {}).setdefault(layer, {})[pos[e["id"]] + w] = c[r]
+                r += 1
+            pos[e["id"]] += len(e["tokens"])
+        assert r == logits.shape[0]
+        for rid in st["end"]:
+            engine.end_sequence(slots.pop(rid))
+        engine.cache.check_invariants()
+    return rows, routes
+
+
+def check(engine, steps, plain, reqs, dtype, what, loosen=1.0, f32_abs=F32_ABS):
+    """Runs the steps and compares every row with the plain implementation.  32-bit: as it decides itself.
+    bfloat16: taking the run's choices of experts, which must be the plain router's own except at close calls."""
+    layers = plain.routed_layers()
+    rows, routes = run_logged(engine, steps, layers)
     assert rows, "nothing was produced"
-    for (rid, p), got in sorted(rows.items()):
-        want = ref[rid][p]
-        assert np.isfinite(got).all(), f"{what}: non-finite logits at request {rid} position {p}"
-        diff = got.astype(np.float64) - want
-        if dtype == "float32":
-            assert np.abs(diff).max() <= f32_abs * max(1.0, want.std()), \
-                f"{what} [float32]: request {rid} position {p} of {len(ref[rid])}: {np.abs(diff).max():.3e}"
-        else:
-            rms, std = float(np.sqrt(np.mean(diff * diff))), float(want.std())
-            assert rms <= loosen * BF16_RMS * std and np.abs(diff).max() <= loosen * BF16_MAX * std, \
-                f"{what} [bfloat16]: request {rid} position {p} of {len(ref[rid])}: rms {rms / std:.3f}, max {np.abs(diff).max() / std:.3f}"
+    for rid, toks in reqs.items():
+        if not any(k[0] == rid for k in rows):
+            continue
+        forced = None
+        if dtype != "float32" and layers:
+            forced = {l: np.stack([routes[rid][l][p] for p in range(len(toks))]) for l in layers}
+        margins, choices = [], []
+        want_all = plain.forward(toks, routes=forced, margins=margins, choices=choices)
+        for l, m, c in zip(layers, margins, choices):      # the run's choices are the plain router's, close calls aside
+            for p in range(len(toks)):
+                if (rid, p) in rows and (dtype == "float32" or m[p] >= CLOSE_CALL):
+                    assert sorted(routes[rid][l][p].tolist()) == sorted(c[p].tolist()), \
+                        f"{what} [{dtype}]: request {rid} position {p} layer {l}: experts {routes[rid][l][p]} for {c[p]}"
+        for p in range(len(toks)):
+            if (rid, p) not in rows:
+                continue
+            got, want = rows[(rid, p)], want_all[p]
+            assert np.isfinite(got).all(), f"{what}: non-finite logits at request {rid} position {p}"
+            diff = got.astype(np.float64) - want
+            if dtype == "float32":
+                assert np.abs(diff).max() <= f32_abs * max(1.0, want.std()), \
+                    f"{what} [float32]: request {rid} position {p} of {len(toks)}: {np.abs(diff).max():.3e}"
+            else:
+                rms, std = float(np.sqrt(np.mean(diff * diff))), float(want.std())
+                assert rms <= loosen * BF16_RMS * std and np.abs(diff).max() <= loosen * BF16_MAX * std, \
+                    f"{what} [bfloat16]: request {rid} position {p} of {len(toks)}: rms {rms / std:.3f}, max {np.abs(diff).max() / std:.3f}"
 
 
 # ------------------------------------------------------------------ kernels alone
@@ -156,6 +213,8 @@ def test_convolution_rotation_blend_and_cache_write(dtype, H, G, D, V, taps, rot
         outs.append([t.cpu().float() for t in (q, kc, vc, own, st)])
     tol = 2e-5 if dtype == torch.float32 else 5e-2
     for name, a, b in zip(("q", "k pages", "v pages", "own values", "state"), *outs):
+        if a.numel() == 0:
+            continue
         assert (a - b).abs().max() < (2e-5 if name in ("own values", "state") else tol), name
 
 
@@ -294,15 +353,15 @@ def test_replays_agree_with_plain(folders, plains, name, dtype):
     another (slots, pages and states used again); prompts in portions down to two tokens and one, alone
     and in mixed batches."""
     reqs = requests_for(LG[name]["vocab"], (1, 7, 64, 150, 65, 33, 290), seed=3)
-    ref = {rid: plains[name].forward(toks) for rid, toks in reqs.items()}
     ids = list(reqs)
     eng = engine_for(folders[name], dtype)
-    compare(run_steps(eng, whole_steps(reqs)), ref, dtype, f"{name} whole")
-    compare(run_steps(eng, tail_steps(reqs, tail=80)), ref, dtype, f"{name} last 80 one by one")
-    compare(run_steps(eng, batch_steps(reqs, [ids[:4], ids[4:]])), ref, dtype, f"{name} unequal batches")
-    compare(run_steps(eng, chunk_steps(reqs, [ids[:3], ids[3:]])), ref, dtype, f"{name} portions in batches")
-    compare(run_steps(eng, chunk_steps(reqs, [[r] for r in ids], sizes=(2,))), ref, dtype, f"{name} portions of 2")
-    compare(run_steps(eng, chunk_steps(reqs, [[r] for r in ids], sizes=(129, 3, 64))), ref, dtype, f"{name} portions of 129")
+    plain = plains[name]
+    check(eng, whole_steps(reqs), plain, reqs, dtype, f"{name} whole")
+    check(eng, tail_steps(reqs, tail=80), plain, reqs, dtype, f"{name} last 80 one by one")
+    check(eng, batch_steps(reqs, [ids[:4], ids[4:]]), plain, reqs, dtype, f"{name} unequal batches")
+    check(eng, chunk_steps(reqs, [ids[:3], ids[3:]]), plain, reqs, dtype, f"{name} portions in batches")
+    check(eng, chunk_steps(reqs, [[r] for r in ids], sizes=(2,)), plain, reqs, dtype, f"{name} portions of 2")
+    check(eng, chunk_steps(reqs, [[r] for r in ids], sizes=(129, 3, 64)), plain, reqs, dtype, f"{name} portions of 129")
     assert not eng.cache.live_slots()
 
 
@@ -314,15 +373,14 @@ def test_configurations_drawn_at_random(tmp_path, seed):
     folder = write_lagedra(str(tmp_path / "m"), raw, seed=seed)
     plain = pl.PlainLagedra.from_folder(folder)
     reqs = requests_for(raw["vocab"], (1, 9, 70, 200, 131), seed=seed)
-    ref = {rid: plain.forward(toks) for rid, toks in reqs.items()}
     ids = list(reqs)
     for dtype in ("float32", "bfloat16"):
         eng = engine_for(folder, dtype)
         what = f"random configuration {seed} ({json.dumps(raw)[:300]})"
-        compare(run_steps(eng, whole_steps(reqs)), ref, dtype, what + " whole", SHARP)
-        compare(run_steps(eng, tail_steps(reqs, tail=33)), ref, dtype, what + " one by one", SHARP)
-        compare(run_steps(eng, batch_steps(reqs, [ids[:3], ids[3:]])), ref, dtype, what + " batches", SHARP)
-        compare(run_steps(eng, chunk_steps(reqs, [ids[:2], ids[2:]])), ref, dtype, what + " portions", SHARP)
+        check(eng, whole_steps(reqs), plain, reqs, dtype, what + " whole", SHARP)
+        check(eng, tail_steps(reqs, tail=33), plain, reqs, dtype, what + " one by one", SHARP)
+        check(eng, batch_steps(reqs, [ids[:3], ids[3:]]), plain, reqs, dtype, what + " batches", SHARP)
+        check(eng, chunk_steps(reqs, [ids[:2], ids[2:]]), plain, reqs, dtype, what + " portions", SHARP)
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
@@ -334,10 +392,9 @@ def test_sharp_attention_over_windows_and_long_decoding(tmp_path, dtype):
     folder = write_lagedra(str(tmp_path / "sharp"), raw, seed=21, sharpen=4.0 if dtype == "float32" else 2.0)
     plain = pl.PlainLagedra.from_folder(folder)
     reqs = {"long": random_tokens(300, 400, 77)}
-    ref = {"long": plain.forward(reqs["long"])}
     eng = engine_for(folder, dtype, max_tokens=64 * 16)
-    compare(run_steps(eng, whole_steps(reqs)), ref, dtype, "sharp whole", SHARP, 1e-3)
-    compare(run_steps(eng, tail_steps(reqs, tail=150)), ref, dtype, "sharp 250 + 150 one by one", SHARP, 1e-3)
+    check(eng, whole_steps(reqs), plain, reqs, dtype, "sharp whole", SHARP, 1e-3)
+    check(eng, tail_steps(reqs, tail=150), plain, reqs, dtype, "sharp 250 + 150 one by one", SHARP, 1e-3)
 
 
 def test_greedy_generation_through_the_entry_point(folders, plains):
@@ -400,4 +457,5 @@ def test_programs(folders, plains, tmp_path):
     finally:
         if p.poll() is None:
             p.kill()
-    compare(rows, ref, "float32", "trace_run")
+    for (rid, p), got in rows.items():
+        assert np.abs(got - ref[rid][p]).max() <= F32_ABS * max(1.0, ref[rid][p].std()), f"trace_run: request {rid} position {p}"
