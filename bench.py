@@ -68,12 +68,13 @@ def parse():
                     help="cache size in tokens (default: batch x context, or what fits in free memory if less)")
     ap.add_argument("--no-graph", action="store_true")
     ap.add_argument("--only", choices=["decode", "prefill"], help="run one part (for profiles); prints no JSON line")
-    ap.add_argument("--design", choices=["tabezen"], default=None,
+    ap.add_argument("--design", choices=["tabezen", "lagedra"], default=None,
                     help="instead of the default workload: prefill and decode of this design at a few layer sizes "
                          "beside the Qwen2 decoder of the same width, depth and feed-forward size, kernel by kernel")
     ap.add_argument("--design-sizes", default="small,medium", help="which of the design's sizes to run")
-    ap.add_argument("--design-model", default="tabezen", choices=["tabezen", "qwen2"],
-                    help="with --design and --only: which of the two models runs the one part (for profiles)")
+    ap.add_argument("--design-model", default=None, choices=["tabezen", "lagedra", "qwen2"],
+                    help="with --design and --only: which of the two models runs the one part (for profiles; "
+                         "default: the design itself)")
     return ap.parse_args()
 
 
@@ -251,6 +252,23 @@ def tabezen_config(width, layers, heads, ff, rank=512, dim=128, rot_dim=64, vdim
                 layers=[att if i % 2 == 0 else gru for i in range(layers)])
 
 
+def lagedra_config(width, layers, heads, ff, dim=128, vdim=128, window=1024, experts=8, top=2, vocab=32768, positions=8192):
+    """Linear attention with decay and capped windowed attention in turn (two layers of each in four), dense and
+    routed feed-forwards in turn; the routed ones have `experts` experts of ff / top values, `top` of them a token,
+    so that a token passes as many feed-forward values as in a dense layer of `ff`."""
+    lin = dict(type="lightning", mixer=dict(heads=heads, dim=dim, vdim=vdim,
+                                            decay=[1.0 - 2.0 ** (-5.0 - 3.0 * h / max(1, heads - 1)) for h in range(heads)]))
+    att = dict(type="attention",
+               mixer=dict(heads=heads, kv_heads=max(1, heads // 4), dim=dim, vdim=vdim, scale=dim ** -0.5, softcap=50.0, conv=4,
+                          mask=dict(size=window), v_mix=True,
+                          rot=dict(base=10000.0, dims=dim // 2, scaling=dict(factor=8.0, original=4096, fast=32.0, slow=1.0))))
+    dense = dict(kind="dense", ff=ff)
+    routed = dict(kind="moe", expert=dict(ff=ff // top, limit=7.0),
+                  router=dict(experts=experts, top=top, groups=dict(count=4, keep=2)))
+    return dict(architecture="Lagedra", vocab=vocab, width=width, max_positions=positions, norm=dict(eps=1e-6),
+                layers=[dict(lin if (i // 2) % 2 == 0 else att, mlp=dense if i % 2 == 0 else routed) for i in range(layers)])
+
+
 def qwen2_like(width, layers, heads, ff, vocab=32768):
     """The Qwen2 decoder of the same width, depth, head count and feed-forward size (head size 128)."""
     return dict(QWEN25_7B, num_hidden_layers=layers, hidden_size=width, num_attention_heads=heads,
@@ -262,6 +280,9 @@ DESIGN_SIZES = {
     "small": dict(width=2048, layers=4, heads=16, ff=8192),
     "medium": dict(width=4096, layers=4, heads=32, ff=14336),
 }
+
+
+DESIGN_CONFIGS = {"tabezen": tabezen_config, "lagedra": lagedra_config, "qwen2": qwen2_like}
 
 
 def traced_step(eng, slots, toks, want):
@@ -342,24 +363,25 @@ def run_design(a) -> int:
     if a.only:                               # one part of one model at the first size, for profiles
         from minfer_amd import LLM
         size = DESIGN_SIZES[a.design_sizes.split(",")[0]]
-        cfg = tabezen_config(**size) if a.design_model == "tabezen" else qwen2_like(**size)
+        cfg = DESIGN_CONFIGS[a.design_model or a.design](**size)
         eng = LLM(config=cfg, random_weights=True, weight_seed=0, dtype=dtype, n_ctx=a.context, n_slots=a.batch).engine
         if a.only == "decode":
             r = run_decode(eng, cfg, a.batch, a.prompt_max, a.steps, a.warmup, not a.no_graph, elem, bytes_fn=lambda *_: 0.0)
-            print(f"{a.design_model} decode batch {a.batch}: {r['tok_s']:.1f} tok/s, {r['ms']:.3f} ms/step")
+            print(f"{a.design_model or a.design} decode batch {a.batch}: {r['tok_s']:.1f} tok/s, {r['ms']:.3f} ms/step")
         else:
             s = run_prefill(eng, cfg, a.prefill_tokens)
-            print(f"{a.design_model} prefill {a.prefill_tokens} tokens: {s * 1e3:.2f} ms, {a.prefill_tokens / s:.0f} tok/s")
+            print(f"{a.design_model or a.design} prefill {a.prefill_tokens} tokens: {s * 1e3:.2f} ms, {a.prefill_tokens / s:.0f} tok/s")
         return 0
     out = {"design": a.design, "dtype": a.dtype, "data": "synthetic", "batch": a.batch, "prompt_max": a.prompt_max,
            "prefill_tokens": a.prefill_tokens, "steps": a.steps, "warmup": a.warmup, "sizes": {}}
     for name in a.design_sizes.split(","):
         size = DESIGN_SIZES[name]
         row = {"size": size}
-        for label, cfg in (("tabezen", tabezen_config(**size)), ("qwen2", qwen2_like(**size))):
+        for label in (a.design, "qwen2"):
             print(f"{name}: {label} ...", file=sys.stderr, flush=True)
-            row[label] = design_point(cfg, a, dtype, elem)
-            row[label]["attention"] = attention_rooflines(size, a, row[label], label == "tabezen")
+            row[label] = design_point(DESIGN_CONFIGS[label](**size), a, dtype, elem)
+            if a.design == "tabezen":
+                row[label]["attention"] = attention_rooflines(size, a, row[label], label == "tabezen")
         out["sizes"][name] = row
     print(json.dumps(out))
     return 0

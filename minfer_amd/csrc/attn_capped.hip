@@ -10,8 +10,8 @@
 //   s_j = cap tanh((q . k_j) scale temp[h] / cap), keys j with 0 <= p - j < window, ordinary softmax,
 //   o = sum_j p_j v_j.
 //
-// `qkv_conv_prep_kernel`: one workgroup per token; convolution of the whole q|k|v row into LDS,
-// then rotation, blending, the cache write and q rounded to the run type.
+// `qkv_conv_prep_kernel`: one workgroup per (token, head of q, k or v); convolution of the head's channels
+// into LDS, then rotation, blending, the cache write and q rounded to the run type.
 // `conv_state_update_kernel`: behind it, the sequences' new last rows.
 // `capped_attn_kernel`: a workgroup owns (token, kv head, up to 8 query heads of its group, key
 // split) and walks the token's keys 256 at a time: a thread forms the scores of one key for all the
@@ -25,64 +25,66 @@
 #define MF_CONV_MAX_TAPS 16
 
 // ------------------------------------------------------------------ preparation
+// A workgroup owns (token, head): a query head, a key head or a value head of the q|k|v row.
 template <typename T>
-__global__ __launch_bounds__(256) void qkv_conv_prep_kernel(
+__global__ __launch_bounds__(128) void qkv_conv_prep_kernel(
     const float* __restrict__ qkv, const float* __restrict__ conv_w, int taps, const float* __restrict__ conv_state,
     const int* __restrict__ cu_seqlens, const int* __restrict__ seq_of_tok, const int* __restrict__ slot_ids,
     const int* __restrict__ positions, const float* __restrict__ cos_t, const float* __restrict__ sin_t, int rot,
     float lambda, const float* __restrict__ v_first, float* __restrict__ v_own, const int* __restrict__ page_table,
     int pt_stride, T* __restrict__ q_out, T* __restrict__ kc, T* __restrict__ vc, int H, int G, int D, int V,
     int write_cache) {
-  extern __shared__ float y[];      // the convolved row
-  const int t = blockIdx.x;
+  extern __shared__ float y[];      // the head's convolved values
+  const int t = blockIdx.x, unit = blockIdx.y;
   const int C = H * D + G * D + G * V;
+  const int kind = unit < H ? 0 : (unit < H + G ? 1 : 2);       // query, key, value
+  const int head = kind == 0 ? unit : (kind == 1 ? unit - H : unit - H - G);
+  const int width = kind == 2 ? V : D;
+  const int c0 = kind == 0 ? head * D : (kind == 1 ? H * D + head * D : H * D + G * D + head * V);
   const int b = seq_of_tok[t];
   const int i = t - cu_seqlens[b];  // index of the token inside its sequence's part of the step
-  const float* row = qkv + (size_t)t * C;
+  const float* row = qkv + (size_t)t * C + c0;
   if (conv_w) {
-    const float* st = taps > 1 ? conv_state + (size_t)slot_ids[b] * (taps - 1) * C : nullptr;
-    for (int c = threadIdx.x; c < C; c += 256) {
+    const float* st = taps > 1 ? conv_state + (size_t)slot_ids[b] * (taps - 1) * C + c0 : nullptr;
+    for (int e = threadIdx.x; e < width; e += 128) {
       float a = 0.f;
       for (int j = 0; j < taps; ++j) {
         const int back = taps - 1 - j;          // this tap reads the row `back` tokens before the token
-        const float u = back <= i ? row[c - (ptrdiff_t)back * C] : st[(size_t)(i + j) * C + c];
-        a = fmaf(conv_w[(size_t)c * taps + j], u, a);
+        const float u = back <= i ? row[e - (ptrdiff_t)back * C] : st[(size_t)(i + j) * C + e];
+        a = fmaf(conv_w[(size_t)(c0 + e) * taps + j], u, a);
       }
-      y[c] = a;
+      y[e] = a;
     }
   } else {
-    for (int c = threadIdx.x; c < C; c += 256) y[c] = row[c];
+    for (int e = threadIdx.x; e < width; e += 128) y[e] = row[e];
   }
   __syncthreads();
   const int p = positions[t];
-  const int half = rot / 2;
-  const float* cs = cos_t + (size_t)p * half;
-  const float* sn = sin_t + (size_t)p * half;
   const int page = write_cache ? page_table[(size_t)b * pt_stride + p / MF_PAGE] : 0;
   const int in_page = p % MF_PAGE;
-  const int nq = H * D, nk = G * D;
-  for (int c = threadIdx.x; c < nq + nk; c += 256) {
-    const int e = c < nq ? c % D : (c - nq) % D;
-    float v = y[c];
-    if (e < half) v = v * cs[e] - y[c + half] * sn[e];
-    else if (e < rot) v = v * cs[e - half] + y[c - half] * sn[e - half];
-    if (c < nq) {
-      q_out[(size_t)t * nq + c] = from_f32<T>(v);
-    } else if (write_cache) {
-      const int g = (c - nq) / D;
-      kc[(((size_t)page * G + g) * MF_PAGE + in_page) * D + e] = from_f32<T>(v);
+  if (kind < 2) {
+    const int half = rot / 2;
+    const float* cs = cos_t + (size_t)p * half;
+    const float* sn = sin_t + (size_t)p * half;
+    for (int e = threadIdx.x; e < D; e += 128) {
+      float v = y[e];
+      if (e < half) v = v * cs[e] - y[e + half] * sn[e];
+      else if (e < rot) v = v * cs[e - half] + y[e - half] * sn[e - half];
+      if (kind == 0) q_out[(size_t)t * H * D + head * D + e] = from_f32<T>(v);
+      else if (write_cache) kc[(((size_t)page * G + head) * MF_PAGE + in_page) * D + e] = from_f32<T>(v);
     }
+    return;
   }
-  for (int c = threadIdx.x; c < G * V; c += 256) {
-    float v = y[nq + nk + c];
+  for (int e = threadIdx.x; e < V; e += 128) {
+    const int c = head * V + e;
+    float v = y[e];
     if (v_own) v_own[(size_t)t * G * V + c] = v;
     if (v_first) v = (1.0f - lambda) * v + lambda * v_first[(size_t)t * G * V + c];
     if (write_cache) {
-      const int g = c / V, e = c % V;
       if (sizeof(T) == 2)      // bfloat16 pages keep V transposed in two halves of 32 keys
-        vc[((((size_t)page * G + g) * 2 + in_page / 32) * V + e) * 32 + in_page % 32] = from_f32<T>(v);
+        vc[((((size_t)page * G + head) * 2 + in_page / 32) * V + e) * 32 + in_page % 32] = from_f32<T>(v);
       else
-        vc[(((size_t)page * G + g) * MF_PAGE + in_page) * V + e] = from_f32<T>(v);
+        vc[(((size_t)page * G + head) * MF_PAGE + in_page) * V + e] = from_f32<T>(v);
     }
   }
 }
@@ -139,8 +141,9 @@ __global__ __launch_bounds__(256) void capped_attn_kernel(
   const int p = positions[t];
   const int* pt = page_table + (size_t)seq_of_tok[t] * pt_stride;
   const int lo = window > 0 ? max(0, p - window + 1) : 0;
-  const int j_begin = max(lo, split * split_len);
-  const int j_end = min(p + 1, (split + 1) * split_len);
+  // a windowed token's splits start at its window's first key, so that all of them have keys
+  const int j_begin = lo + split * split_len;
+  const int j_end = min(p + 1, j_begin + split_len);
 
   for (int i = threadIdx.x; i < gcount * D; i += 256)
     sq[i] = to_f32(q[((size_t)t * nh + h0) * D + i]);
@@ -284,25 +287,18 @@ MF_API int mf_qkv_conv_prep(const float* qkv, const float* conv_w, int taps, flo
   if (n_tok <= 0) return 0;
   const int C = H * D + G * D + G * V;
   if (H <= 0 || G <= 0 || D <= 0 || V <= 0 || rot < 0 || rot % 2 || rot > D || taps < 1 || taps > MF_CONV_MAX_TAPS ||
-      (taps > 1 && (!conv_w || !conv_state)) || (size_t)C * sizeof(float) > 160 * 1024 - 1024)
+      (taps > 1 && (!conv_w || !conv_state)) || D > 8192 || V > 8192)
     return (int)hipErrorInvalidValue;
-  const size_t lds = (size_t)C * sizeof(float);
+  const size_t lds = (size_t)(D > V ? D : V) * sizeof(float);
+  const dim3 grid(n_tok, H + 2 * G);
   int rc;
   if (is_bf16) {
-    if (lds > 48 * 1024) {
-      rc = (int)hipFuncSetAttribute((const void*)qkv_conv_prep_kernel<bf16>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-      if (rc) return rc;
-    }
-    qkv_conv_prep_kernel<bf16><<<n_tok, 256, lds, stream>>>(qkv, conv_w, taps, conv_state, cu_seqlens, seq_of_tok, slot_ids,
+    qkv_conv_prep_kernel<bf16><<<grid, 128, lds, stream>>>(qkv, conv_w, taps, conv_state, cu_seqlens, seq_of_tok, slot_ids,
                                                             positions, cos_t, sin_t, rot, lambda, v_first, v_own, page_table,
                                                             pt_stride, (bf16*)q_out, (bf16*)kc, (bf16*)vc, H, G, D, V,
                                                             write_cache);
   } else {
-    if (lds > 48 * 1024) {
-      rc = (int)hipFuncSetAttribute((const void*)qkv_conv_prep_kernel<float>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-      if (rc) return rc;
-    }
-    qkv_conv_prep_kernel<float><<<n_tok, 256, lds, stream>>>(qkv, conv_w, taps, conv_state, cu_seqlens, seq_of_tok, slot_ids,
+    qkv_conv_prep_kernel<float><<<grid, 128, lds, stream>>>(qkv, conv_w, taps, conv_state, cu_seqlens, seq_of_tok, slot_ids,
                                                              positions, cos_t, sin_t, rot, lambda, v_first, v_own, page_table,
                                                              pt_stride, (float*)q_out, (float*)kc, (float*)vc, H, G, D, V,
                                                              write_cache);

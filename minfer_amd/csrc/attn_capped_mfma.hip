@@ -1,0 +1,220 @@
+// Windowed, capped attention for many query tokens per sequence (prompts and their portions), bfloat16, on
+// the gfx950 matrix cores, for keys of MF_CAPM_D and values of MF_CAPM_V values (multiples of 16, given at
+// compile time: the library is built for a model's sizes).  Semantics as `capped_attn_kernel`:
+// s = cap tanh(q . k scale temp[h] / cap), keys j with 0 <= p - j < window, softmax, o = sum p_j v_j.
+//
+// A wave owns 16 consecutive new tokens of one sequence times RB query heads of one kv head and walks the
+// tokens' keys 32 at a time (half a page), with no LDS and no barrier:
+//   S^T[key][token] = K Q^T      16x16x32 MFMA, A = 16 key rows straight from the cache, B = Q kept in registers
+//   a lane holds, for its token (lane % 16), the scores of keys 4 (lane / 16) + i of both key tiles:
+//   the softmax statistics are per lane, shared by the four lanes of a token through two shuffles
+//   O^T[d][token] += V^T P^T     A = rows of V^T straight from the cache, which stores a page's values
+//   transposed in halves of 32 keys; B = P^T, the scores' own register layout.  The k index of this product
+//   is permuted the same way on both operands: slot 8 g + j stands for key 4 g + j (j < 4) and 16 + 4 g + j - 4.
+// The RB heads share every K and V fragment.  Sums, maxima and outputs are 32-bit; probabilities are rounded
+// to bfloat16 for the second product.  Keys not yet written (behind the sequence's end) may hold anything:
+// their scores are masked and their value columns are zeroed before the product.
+#include "common.h"
+
+#ifndef MF_CAPM_D
+#define MF_CAPM_D 128
+#endif
+#ifndef MF_CAPM_V
+#define MF_CAPM_V 128
+#endif
+
+namespace {
+
+constexpr int D = MF_CAPM_D, V = MF_CAPM_V;
+constexpr int DKS = (D + 31) / 32;     // k steps of the first product
+constexpr int NVT = V / 16;            // output tiles
+static_assert(D % 16 == 0 && V % 16 == 0 && D <= 256 && V <= 256, "sizes the kernel takes");
+
+typedef short short4v __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ float fast_tanh(float y) {
+  // 1 - 2 / (e^(2y) + 1), exact at both ends
+  const float e = __expf(2.0f * y);
+  return 1.0f - 2.0f / (e + 1.0f);
+}
+
+template <int RB>
+__global__ __launch_bounds__(256) void capped_mfma_kernel(
+    const bf16* __restrict__ q, const bf16* __restrict__ kc, const bf16* __restrict__ vc,
+    const int* __restrict__ page_table, int pt_stride, const int* __restrict__ cu_seqlens,
+    const int* __restrict__ start_pos, const int* __restrict__ tile_seq, const int* __restrict__ tile_q0, int n_tiles,
+    const float* __restrict__ temp, bf16* __restrict__ out, int nh, int nk, float scale, float cap, int window) {
+  const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+  const int tile = blockIdx.x * 4 + w;
+  if (tile >= n_tiles) return;
+  const int G = nh / nk;
+  const int n_hc = G / RB;
+  const int hk = blockIdx.y / n_hc;
+  const int h0 = hk * G + (blockIdx.y % n_hc) * RB;
+  const int col = lane & 15, g = lane >> 4;
+
+  const int b = tile_seq[tile], q0 = tile_q0[tile];
+  const int t_first = cu_seqlens[b] + q0;
+  const int n_new = cu_seqlens[b + 1] - cu_seqlens[b];
+  const int rows = min(16, n_new - q0);
+  const int p0 = start_pos[b] + q0;               // position of the tile's first token
+  const int p_last = p0 + rows - 1;
+  const int seq_end = start_pos[b] + n_new;       // keys from here on were never written
+  const int p_mine = p0 + col;                    // this lane's token (rows beyond `rows` are masked out)
+  const bool row_ok = col < rows;
+  const int* pt = page_table + (size_t)b * pt_stride;
+  const int lo = window > 0 ? max(0, p0 - window + 1) : 0;
+
+  // Q fragments: token `col`, values 32 ks + 8 g .. + 8 of head h0 + r
+  bf16x8 qf[RB][DKS];
+#pragma unroll
+  for (int r = 0; r < RB; ++r)
+#pragma unroll
+    for (int ks = 0; ks < DKS; ++ks) {
+      const int d = ks * 32 + g * 8;
+      bf16x8 v = {};
+      if (row_ok && d < D) v = *(const bf16x8*)(q + ((size_t)(t_first + col) * nh + h0 + r) * D + d);
+      qf[r][ks] = v;
+    }
+  float sc[RB];
+#pragma unroll
+  for (int r = 0; r < RB; ++r) sc[r] = scale * temp[h0 + r];
+  const float inv_cap = cap > 0.f ? 1.0f / cap : 0.f;
+
+  floatx4 oacc[RB][NVT];
+  float m[RB], l[RB];
+#pragma unroll
+  for (int r = 0; r < RB; ++r) {
+    m[r] = -INFINITY;
+    l[r] = 0.f;
+#pragma unroll
+    for (int c = 0; c < NVT; ++c) oacc[r][c] = floatx4{0.f, 0.f, 0.f, 0.f};
+  }
+
+  for (int kb = lo & ~31; kb <= p_last; kb += 32) {
+    const int page = pt[kb / MF_PAGE];
+    const int in_page = kb % MF_PAGE;              // 0 or 32
+    // K fragments of both key tiles: key row `col` (+ 16), values 32 ks + 8 g .. + 8
+    const bf16* kbase = kc + (((size_t)page * nk + hk) * MF_PAGE + in_page + col) * D + g * 8;
+    bf16x8 kf[2][DKS];
+#pragma unroll
+    for (int a = 0; a < 2; ++a)
+#pragma unroll
+      for (int ks = 0; ks < DKS; ++ks) {
+        bf16x8 v = {};
+        if (ks * 32 + g * 8 < D) v = *(const bf16x8*)(kbase + (size_t)a * 16 * D + ks * 32);
+        kf[a][ks] = v;
+      }
+    // which of this lane's 8 keys its token sees: slot j < 4: key kb + 4 g + j, else kb + 16 + 4 g + j - 4
+    bool seen[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const int key = kb + (j < 4 ? 4 * g + j : 16 + 4 * g + j - 4);
+      seen[j] = row_ok && key <= p_mine && (window <= 0 || p_mine - key < window);
+    }
+    bf16x8 pf[RB];
+#pragma unroll
+    for (int r = 0; r < RB; ++r) {
+      floatx4 s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int ks = 0; ks < DKS; ++ks) {
+        s0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[0][ks], qf[r][ks], s0, 0, 0, 0);
+        s1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[1][ks], qf[r][ks], s1, 0, 0, 0);
+      }
+      float x[8];
+      float mx = -INFINITY;
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        float y = (j < 4 ? s0[j] : s1[j - 4]) * sc[r];
+        if (cap > 0.f) y = cap * fast_tanh(y * inv_cap);
+        x[j] = seen[j] ? y : -INFINITY;
+        mx = fmaxf(mx, x[j]);
+      }
+      mx = fmaxf(mx, __shfl_xor(mx, 16, MF_WAVE));
+      mx = fmaxf(mx, __shfl_xor(mx, 32, MF_WAVE));
+      const float m_new = fmaxf(m[r], mx);
+      const float corr = m[r] == -INFINITY ? 1.f : __expf(m[r] - m_new);
+      float sum = 0.f;
+      bf16x8 p;
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const float pe = seen[j] ? __expf(x[j] - m_new) : 0.f;
+        sum += pe;
+        p[j] = (bf16)pe;
+      }
+      pf[r] = p;
+      l[r] = l[r] * corr + sum;
+      m[r] = m_new;
+#pragma unroll
+      for (int c = 0; c < NVT; ++c) oacc[r][c] *= corr;
+    }
+    // V^T fragments: value row 16 c + col, keys 4 g .. + 4 and 16 + 4 g .. + 4 of this half page
+    const bf16* vbase = vc + ((((size_t)page * nk + hk) * 2 + in_page / 32) * V + col) * 32 + 4 * g;
+    const bool tail = kb + 32 > seq_end;           // some of these keys were never written
+#pragma unroll
+    for (int c = 0; c < NVT; ++c) {
+      const bf16* vp = vbase + (size_t)c * 16 * 32;
+      short4v lo4 = *(const short4v*)vp, hi4 = *(const short4v*)(vp + 16);
+      if (tail) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          if (kb + 4 * g + j >= seq_end) lo4[j] = 0;
+          if (kb + 16 + 4 * g + j >= seq_end) hi4[j] = 0;
+        }
+      }
+      typedef short short8v __attribute__((ext_vector_type(8)));
+      const short8v both = {lo4[0], lo4[1], lo4[2], lo4[3], hi4[0], hi4[1], hi4[2], hi4[3]};
+      const bf16x8 vf = __builtin_bit_cast(bf16x8, both);
+#pragma unroll
+      for (int r = 0; r < RB; ++r) oacc[r][c] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pf[r], oacc[r][c], 0, 0, 0);
+    }
+  }
+
+  // O^T[d = 16 c + 4 g + i][token col] -> out[token][head][d]
+#pragma unroll
+  for (int r = 0; r < RB; ++r) {
+    float L = l[r];
+    L += __shfl_xor(L, 16, MF_WAVE);
+    L += __shfl_xor(L, 32, MF_WAVE);
+    const float inv = L > 0.f ? 1.0f / L : 0.f;
+    if (row_ok) {
+      bf16* o = out + ((size_t)(t_first + col) * nh + h0 + r) * V + 4 * g;
+#pragma unroll
+      for (int c = 0; c < NVT; ++c) {
+        bf16x4 v4;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) v4[i] = (bf16)(oacc[r][c][i] * inv);
+        *(bf16x4*)(o + c * 16) = v4;
+      }
+    }
+  }
+}
+
+}  // namespace
+
+MF_API int mf_capped_mfma_sizes(int* d, int* v) {
+  *d = D;
+  *v = V;
+  return 0;
+}
+
+// tiles: blocks of 16 consecutive new tokens of a sequence (tile_seq, tile_q0), n_tiles of them
+MF_API int mf_capped_mfma(const void* q, const void* kc, const void* vc, const int* page_table, int pt_stride,
+                          const int* cu_seqlens, const int* start_pos, const int* tile_seq, const int* tile_q0,
+                          int n_tiles, const float* temp, void* out, int nh, int nk, int d, int v, float scale, float cap,
+                          int window, hipStream_t stream) {
+  if (n_tiles <= 0) return 0;
+  if (d != D || v != V || nk <= 0 || nh % nk || !temp) return (int)hipErrorInvalidValue;
+  const int G = nh / nk;
+  const int rb = G % 4 == 0 ? 4 : (G % 2 == 0 ? 2 : 1);
+  dim3 grid((n_tiles + 3) / 4, nk * (G / rb));
+#define MF_GO(RB)                                                                                                          \
+  capped_mfma_kernel<RB><<<grid, 256, 0, stream>>>((const bf16*)q, (const bf16*)kc, (const bf16*)vc, page_table, pt_stride, \
+                                                   cu_seqlens, start_pos, tile_seq, tile_q0, n_tiles, temp, (bf16*)out, nh, \
+                                                   nk, scale, cap, window)
+  if (rb == 4) MF_GO(4);
+  else if (rb == 2) MF_GO(2);
+  else MF_GO(1);
+#undef MF_GO
+  return mf_launch_status();
+}

@@ -659,11 +659,17 @@ __global__ __launch_bounds__(256) void weighted_sum_kernel(WsumPtrs src, int n, 
   const int r = blockIdx.x;
   const int ri = row_idx ? row_idx[r] : r;
   float* o = out + (size_t)r * d;
-  for (int i = threadIdx.x; i < d; i += 256) {
-    float a = add ? o[i] : 0.f;
-    for (int j = 0; j < n; ++j) a = fmaf(w[j], src.p[j][(size_t)(j < n_indexed ? ri : r) * d + i], a);
-    o[i] = a;
-  }
+  const int i = blockIdx.y * 256 + threadIdx.x;
+  if (i >= d) return;
+  float v[MF_WSUM_MAX];
+#pragma unroll
+  for (int j = 0; j < MF_WSUM_MAX; ++j)          // all loads first: one trip to memory
+    v[j] = j < n ? src.p[j][(size_t)(j < n_indexed ? ri : r) * d + i] : 0.f;
+  float a = add ? o[i] : 0.f;
+#pragma unroll
+  for (int j = 0; j < MF_WSUM_MAX; ++j)
+    if (j < n) a = fmaf(w[j], v[j], a);
+  o[i] = a;
 }
 
 // `ptrs`: host array of n device pointers
@@ -676,7 +682,7 @@ MF_API int mf_weighted_sum(const void* const* ptrs, int n, int n_indexed, const 
     const int m = n - j0 < MF_WSUM_MAX ? n - j0 : MF_WSUM_MAX;
     for (int j = 0; j < MF_WSUM_MAX; ++j) a.p[j] = j < m ? (const float*)ptrs[j0 + j] : nullptr;
     const int idx = n_indexed - j0 < 0 ? 0 : (n_indexed - j0 > m ? m : n_indexed - j0);
-    weighted_sum_kernel<<<rows, 256, 0, stream>>>(a, m, idx, row_idx, w + j0, out, d, j0 > 0 ? 1 : 0);
+    weighted_sum_kernel<<<dim3(rows, (d + 255) / 256), 256, 0, stream>>>(a, m, idx, row_idx, w + j0, out, d, j0 > 0 ? 1 : 0);
     const int rc = mf_launch_status();
     if (rc) return rc;
   }

@@ -1,6 +1,6 @@
 // Mixture of experts: the router's choice and the experts' activation.
 //
-// Router: scores = softmax of the router's 32-bit logits over all experts; the experts form `n_groups`
+// Router: logits = Wr x in 32-bit, scores = their softmax over all experts; the experts form `n_groups`
 // equal groups of neighbours, a group's score is its best expert's, only experts of the `keep` best
 // groups can be chosen; the `top` best of those are chosen (ties go to the lower index) and weighted
 // by their scores over the sum of the chosen scores (+ 1e-20).  One wave per token.
@@ -25,21 +25,63 @@ __device__ __forceinline__ void wave_argmax(float& v, int& idx) {
   }
 }
 
-__global__ __launch_bounds__(64) void moe_route_kernel(const float* __restrict__ logits, float* __restrict__ dense,
-                                                       int* __restrict__ chosen, float* __restrict__ weights, int E,
-                                                       int n_groups, int keep, int top) {
+// what one wave needs to see its own earlier LDS writes (the deciding part runs in one wave)
+#define MF_WAVE_SYNC()                                     \
+  do {                                                     \
+    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront"); \
+    __builtin_amdgcn_wave_barrier();                       \
+  } while (0)
+
+__device__ __forceinline__ void load4(const bf16* __restrict__ p, float (&d)[4]) {
+  alignas(8) bf16 raw[4];
+  *(uint2*)raw = *(const uint2*)p;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) d[i] = (float)raw[i];
+}
+__device__ __forceinline__ void load4(const float* __restrict__ p, float (&d)[4]) {
+  const float4 v = *(const float4*)p;
+  d[0] = v.x; d[1] = v.y; d[2] = v.z; d[3] = v.w;
+}
+
+// x [tokens][K] in the run type, router [E][K] float32: a workgroup per token; its four waves form the E
+// logits (a wave an expert at a time, lanes over K in runs of 4, sums in 32-bit), then the first wave decides.
+template <typename XT>
+__global__ __launch_bounds__(256) void moe_route_kernel(const XT* __restrict__ x, const float* __restrict__ router, int K,
+                                                       float* __restrict__ dense, int* __restrict__ chosen,
+                                                       float* __restrict__ weights, int E, int n_groups, int keep,
+                                                       int top) {
   __shared__ float s[MF_MOE_MAX_EXPERTS], ms[MF_MOE_MAX_EXPERTS], gs[MF_MOE_MAX_EXPERTS];
-  const int t = blockIdx.x, lane = threadIdx.x;
-  const float* z = logits + (size_t)t * E;
+  const int t = blockIdx.x, lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+  const XT* xr = x + (size_t)t * K;
+  for (int e = wv; e < E; e += 4) {
+    const float* wr = router + (size_t)e * K;
+    float a = 0.f;
+    if (K % 4 == 0) {
+#pragma unroll 8
+      for (int i = lane * 4; i < K; i += 256) {
+        float w4[4], x4[4];
+        load4(wr + i, w4);
+        load4(xr + i, x4);
+#pragma unroll
+        for (int q = 0; q < 4; ++q) a = fmaf(w4[q], x4[q], a);
+      }
+    } else {
+      for (int i = lane; i < K; i += 64) a = fmaf(wr[i], to_f32(xr[i]), a);
+    }
+    a = wave_sum(a);
+    if (lane == 0) s[e] = a;
+  }
+  __syncthreads();
+  if (wv != 0) return;              // from here on one wave: MF_WAVE_SYNC where the block form has a barrier
   float mx = -INFINITY;
-  for (int e = lane; e < E; e += 64) mx = fmaxf(mx, z[e]);
+  for (int e = lane; e < E; e += 64) mx = fmaxf(mx, s[e]);
   mx = wave_max(mx);
   float sum = 0.f;
-  for (int e = lane; e < E; e += 64) { const float x = expf(z[e] - mx); s[e] = x; sum += x; }
+  for (int e = lane; e < E; e += 64) { const float v = expf(s[e] - mx); s[e] = v; sum += v; }
   sum = wave_sum(sum);
-  __syncthreads();
+  MF_WAVE_SYNC();
   for (int e = lane; e < E; e += 64) { s[e] = s[e] / sum; dense[(size_t)t * E + e] = 0.f; }
-  __syncthreads();
+  MF_WAVE_SYNC();
   const int per = E / n_groups;
   for (int g = lane; g < n_groups; g += 64) {
     float b = -1.f;
@@ -47,17 +89,17 @@ __global__ __launch_bounds__(64) void moe_route_kernel(const float* __restrict__
     gs[g] = b;
   }
   for (int e = lane; e < E; e += 64) ms[e] = -1.f;
-  __syncthreads();
+  MF_WAVE_SYNC();
   for (int k = 0; k < keep; ++k) {
     float b = -2.f;
     int bi = 0x7fffffff;
     for (int g = lane; g < n_groups; g += 64)
       if (gs[g] > b) { b = gs[g]; bi = g; }
     wave_argmax(b, bi);
-    __syncthreads();
+    MF_WAVE_SYNC();
     if (lane == 0) gs[bi] = -3.f;
     for (int i = lane; i < per; i += 64) ms[bi * per + i] = s[bi * per + i];
-    __syncthreads();
+    MF_WAVE_SYNC();
   }
   float wsum = 0.f;
   int mine = -1;          // lane k keeps the k-th choice (top <= 64)
@@ -67,11 +109,11 @@ __global__ __launch_bounds__(64) void moe_route_kernel(const float* __restrict__
     for (int e = lane; e < E; e += 64)
       if (ms[e] > b) { b = ms[e]; bi = e; }
     wave_argmax(b, bi);
-    __syncthreads();
+    MF_WAVE_SYNC();
     if (lane == 0) ms[bi] = -3.f;
     if (lane == k) mine = bi;
     wsum += s[bi];
-    __syncthreads();
+    MF_WAVE_SYNC();
   }
   if (lane < top) {
     const float wgt = s[mine] / (wsum + 1e-20f);
@@ -103,60 +145,157 @@ __global__ __launch_bounds__(256) void moe_act_kernel(const float* __restrict__ 
 }
 
 // ------------------------------------------------------------------ few tokens: the chosen experts only
+// Every chosen expert's matrices are read once, however many of the step's tokens chose it.  The step's
+// (token, choice) pairs, at most MF_MOE_SPARSE_PAIRS of at most MF_MOE_SPARSE_TOKENS tokens, are found by
+// the waves themselves: lane i holds the expert of pair i (and of pair i + 64), and a ballot gives the pairs
+// of an expert as a bit mask.  An expert has at most one pair per token.
+#define MF_MOE_SPARSE_PAIRS 128
+#define MF_MOE_SPARSE_TOKENS 16
+
+__device__ __forceinline__ void load8(const bf16* __restrict__ p, bool vec, int left, float (&dst)[8]) {
+  if (vec && left >= 8) {
+    alignas(16) bf16 raw[8];
+    *(uint4*)raw = *(const uint4*)p;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) dst[i] = (float)raw[i];
+  } else {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) dst[i] = i < left ? (float)p[i] : 0.f;
+  }
+}
+__device__ __forceinline__ void load8(const float* __restrict__ p, bool vec, int left, float (&dst)[8]) {
+  if (vec && left >= 8) {
+    const float4 a = *(const float4*)p, b = *(const float4*)(p + 4);
+    dst[0] = a.x; dst[1] = a.y; dst[2] = a.z; dst[3] = a.w; dst[4] = b.x; dst[5] = b.y; dst[6] = b.z; dst[7] = b.w;
+  } else {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) dst[i] = i < left ? p[i] : 0.f;
+  }
+}
+
+// the lowest pair of the masks, taken off them
+__device__ __forceinline__ int next_pair(unsigned long long& m0, unsigned long long& m1) {
+  if (m0) { const int i = __builtin_ctzll(m0); m0 &= m0 - 1; return i; }
+  const int i = __builtin_ctzll(m1); m1 &= m1 - 1; return 64 + i;
+}
+
 // gate_up [E][2 F][K], x [tokens][K] -> y [tokens][top][F] (activation applied, not weighted).
-// A wave per (token, choice, f): both rows of the pair, lanes over K.
+// A wave owns (expert, f): lanes over K in runs of 8; the gate row and the up row f are read once and
+// meet the x rows of the expert's tokens.
 template <typename WT>
 __global__ __launch_bounds__(256) void moe_sparse_up_kernel(const WT* __restrict__ x, const WT* __restrict__ gate_up,
                                                             const int* __restrict__ chosen, WT* __restrict__ y,
-                                                            int top, int F, int K, float limit) {
-  const int t = blockIdx.x, k = blockIdx.y;
-  const int f = blockIdx.z * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
-  if (f >= F) return;
-  const int e = chosen[(size_t)t * top + k];
+                                                            int n_pairs, int top, int F, int K, float limit) {
+  const int e = blockIdx.x;
+  const int lane = threadIdx.x & 63;
+  const int f = blockIdx.y * 4 + (threadIdx.x >> 6);
+  const int c0 = lane < n_pairs ? chosen[lane] : -1, c1 = lane + 64 < n_pairs ? chosen[lane + 64] : -1;
+  const unsigned long long mine0 = __ballot(c0 == e), mine1 = __ballot(c1 == e);
+  if (!(mine0 | mine1) || f >= F) return;
   const WT* wg = gate_up + ((size_t)e * 2 * F + f) * K;
   const WT* wu = wg + (size_t)F * K;
-  const WT* xr = x + (size_t)t * K;
-  float g = 0.f, u = 0.f;
-  for (int i = lane; i < K; i += 64) {
-    const float xv = to_f32(xr[i]);
-    g = fmaf(to_f32(wg[i]), xv, g);
-    u = fmaf(to_f32(wu[i]), xv, u);
+  const bool vec = (K * sizeof(WT)) % 16 == 0;
+  float ag[MF_MOE_SPARSE_TOKENS], au[MF_MOE_SPARSE_TOKENS];
+#pragma unroll
+  for (int j = 0; j < MF_MOE_SPARSE_TOKENS; ++j) ag[j] = au[j] = 0.f;
+  for (int k = lane * 8; k < K; k += 512) {
+    float g[8], u[8];
+    load8(wg + k, vec, K - k, g);
+    load8(wu + k, vec, K - k, u);
+    unsigned long long m0 = mine0, m1 = mine1;
+#pragma unroll
+    for (int j = 0; j < MF_MOE_SPARSE_TOKENS; ++j) {
+      if (m0 | m1) {
+        const int pr = next_pair(m0, m1);
+        float xv[8];
+        load8(x + (size_t)(pr / top) * K + k, vec, K - k, xv);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) { ag[j] = fmaf(g[i], xv[i], ag[j]); au[j] = fmaf(u[i], xv[i], au[j]); }
+      }
+    }
   }
-  g = wave_sum(g);
-  u = wave_sum(u);
-  if (lane == 0) y[((size_t)t * top + k) * F + f] = from_f32<WT>(expert_act(g, u, limit));
+  unsigned long long m0 = mine0, m1 = mine1;
+#pragma unroll
+  for (int j = 0; j < MF_MOE_SPARSE_TOKENS; ++j) {
+    if (m0 | m1) {
+      const int pr = next_pair(m0, m1);
+      const float g = wave_sum(ag[j]), u = wave_sum(au[j]);
+      if (lane == 0) y[(size_t)pr * F + f] = from_f32<WT>(expert_act(g, u, limit));
+    }
+  }
 }
 
 // down [N][E F] (the experts' down matrices side by side), y [tokens][top][F]:
-// out[t][n] += sum_k w[t][k] dot(down[n][e_k F .. e_k F + F), y[t][k]), choices added in their order.
+// out[t][n] += sum_k w[t][k] dot(down[n][e_k F .. e_k F + F), y[t][k]), a token's choices added in their order.
+// A wave owns output n: for every expert that has pairs, its part of row n is read once and meets the y rows
+// of the expert's pairs; lane p % 64 keeps pair p's dot product until the tokens' sums are formed.
 template <typename WT>
 __global__ __launch_bounds__(256) void moe_sparse_down_kernel(const WT* __restrict__ y, const WT* __restrict__ down,
                                                               const int* __restrict__ chosen,
                                                               const float* __restrict__ weights, float* __restrict__ out,
-                                                              int top, int E, int F, int N) {
-  const int t = blockIdx.x;
-  const int n = blockIdx.y * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
+                                                              int n_tok, int top, int E, int F, int N) {
+  const int lane = threadIdx.x & 63;
+  const int n = blockIdx.x * 4 + (threadIdx.x >> 6);
   if (n >= N) return;
+  const int n_pairs = n_tok * top;
+  const int c0 = lane < n_pairs ? chosen[lane] : -1, c1 = lane + 64 < n_pairs ? chosen[lane + 64] : -1;
+  const bool vec = (F * sizeof(WT)) % 16 == 0;
+  float dot0 = 0.f, dot1 = 0.f;          // of pair lane, of pair lane + 64
+  for (int i = 0; i < n_pairs; ++i) {
+    const int e = chosen[i];
+    const unsigned long long mine0 = __ballot(c0 == e), mine1 = __ballot(c1 == e);
+    const unsigned long long before0 = i < 64 ? (i ? ~0ull >> (64 - i) : 0ull) : ~0ull;
+    const unsigned long long before1 = i <= 64 ? 0ull : ~0ull >> (128 - i);
+    if ((mine0 & before0) | (mine1 & before1)) continue;       // an earlier pair led this expert
+    const WT* wr = down + (size_t)n * E * F + (size_t)e * F;
+    float acc[MF_MOE_SPARSE_TOKENS];
+#pragma unroll
+    for (int j = 0; j < MF_MOE_SPARSE_TOKENS; ++j) acc[j] = 0.f;
+    for (int k = lane * 8; k < F; k += 512) {
+      float wv[8];
+      load8(wr + k, vec, F - k, wv);
+      unsigned long long m0 = mine0, m1 = mine1;
+#pragma unroll
+      for (int j = 0; j < MF_MOE_SPARSE_TOKENS; ++j) {
+        if (m0 | m1) {
+          const int pr = next_pair(m0, m1);
+          float yv[8];
+          load8(y + (size_t)pr * F + k, vec, F - k, yv);
+#pragma unroll
+          for (int q = 0; q < 8; ++q) acc[j] = fmaf(wv[q], yv[q], acc[j]);
+        }
+      }
+    }
+    unsigned long long m0 = mine0, m1 = mine1;
+#pragma unroll
+    for (int j = 0; j < MF_MOE_SPARSE_TOKENS; ++j) {
+      if (m0 | m1) {
+        const int pr = next_pair(m0, m1);
+        const float v = wave_sum(acc[j]);
+        if (lane == (pr & 63)) { if (pr < 64) dot0 = v; else dot1 = v; }
+      }
+    }
+  }
   float total = 0.f;
   for (int k = 0; k < top; ++k) {
-    const int e = chosen[(size_t)t * top + k];
-    const WT* wr = down + (size_t)n * E * F + (size_t)e * F;
-    const WT* yr = y + ((size_t)t * top + k) * F;
-    float a = 0.f;
-    for (int i = lane; i < F; i += 64) a = fmaf(to_f32(wr[i]), to_f32(yr[i]), a);
-    total = fmaf(weights[(size_t)t * top + k], wave_sum(a), total);
+    const int pr = min(lane, n_tok - 1) * top + k;       // lanes behind the tokens repeat the last one's work
+    const float d0 = __shfl(dot0, pr & 63, MF_WAVE), d1 = __shfl(dot1, pr & 63, MF_WAVE);
+    total = fmaf(weights[pr], pr < 64 ? d0 : d1, total);
   }
-  if (lane == 0) out[(size_t)t * N + n] += total;
+  if (lane < n_tok) out[(size_t)lane * N + n] += total;
 }
 
 // ------------------------------------------------------------------ entry points
-MF_API int mf_moe_route(const float* logits, float* dense, int* chosen, float* weights, int n_tok, int E, int n_groups,
-                        int keep, int top, hipStream_t stream) {
+MF_API int mf_moe_route(const void* x, int x_is_bf16, const float* router, int K, float* dense, int* chosen,
+                        float* weights, int n_tok, int E, int n_groups, int keep, int top, hipStream_t stream) {
   if (n_tok <= 0) return 0;
-  if (E <= 0 || E > MF_MOE_MAX_EXPERTS || n_groups <= 0 || E % n_groups || keep <= 0 || keep > n_groups || top <= 0 ||
+  if (K <= 0 || E <= 0 || E > MF_MOE_MAX_EXPERTS || n_groups <= 0 || E % n_groups || keep <= 0 || keep > n_groups || top <= 0 ||
       top > 64 || top > keep * (E / n_groups))
     return (int)hipErrorInvalidValue;
-  moe_route_kernel<<<n_tok, 64, 0, stream>>>(logits, dense, chosen, weights, E, n_groups, keep, top);
+  if (x_is_bf16)
+    moe_route_kernel<bf16><<<n_tok, 256, 0, stream>>>((const bf16*)x, router, K, dense, chosen, weights, E, n_groups, keep, top);
+  else
+    moe_route_kernel<float><<<n_tok, 256, 0, stream>>>((const float*)x, router, K, dense, chosen, weights, E, n_groups, keep, top);
   return mf_launch_status();
 }
 
@@ -177,18 +316,19 @@ MF_API int mf_moe_sparse(const void* x, const void* gate_up, const void* down, c
                          void* y, float* out, int is_bf16, int n_tok, int top, int E, int F, int K, int N, float limit,
                          hipStream_t stream) {
   if (n_tok <= 0) return 0;
-  if (top <= 0 || E <= 0 || F <= 0 || K <= 0 || N <= 0) return (int)hipErrorInvalidValue;
-  dim3 g1(n_tok, top, (F + 3) / 4), g2(n_tok, (N + 3) / 4);
+  if (top <= 0 || E <= 0 || F <= 0 || K <= 0 || N <= 0 || n_tok > MF_MOE_SPARSE_TOKENS || n_tok * top > MF_MOE_SPARSE_PAIRS)
+    return (int)hipErrorInvalidValue;
+  dim3 g1(E, (F + 3) / 4), g2((N + 3) / 4);
   if (is_bf16) {
-    moe_sparse_up_kernel<bf16><<<g1, 256, 0, stream>>>((const bf16*)x, (const bf16*)gate_up, chosen, (bf16*)y, top, F, K, limit);
+    moe_sparse_up_kernel<bf16><<<g1, 256, 0, stream>>>((const bf16*)x, (const bf16*)gate_up, chosen, (bf16*)y, n_tok * top, top, F, K, limit);
     int rc = mf_launch_status();
     if (rc) return rc;
-    moe_sparse_down_kernel<bf16><<<g2, 256, 0, stream>>>((const bf16*)y, (const bf16*)down, chosen, weights, out, top, E, F, N);
+    moe_sparse_down_kernel<bf16><<<g2, 256, 0, stream>>>((const bf16*)y, (const bf16*)down, chosen, weights, out, n_tok, top, E, F, N);
   } else {
-    moe_sparse_up_kernel<float><<<g1, 256, 0, stream>>>((const float*)x, (const float*)gate_up, chosen, (float*)y, top, F, K, limit);
+    moe_sparse_up_kernel<float><<<g1, 256, 0, stream>>>((const float*)x, (const float*)gate_up, chosen, (float*)y, n_tok * top, top, F, K, limit);
     int rc = mf_launch_status();
     if (rc) return rc;
-    moe_sparse_down_kernel<float><<<g2, 256, 0, stream>>>((const float*)y, (const float*)down, chosen, weights, out, top, E, F, N);
+    moe_sparse_down_kernel<float><<<g2, 256, 0, stream>>>((const float*)y, (const float*)down, chosen, weights, out, n_tok, top, E, F, N);
   }
   return mf_launch_status();
 }

@@ -35,6 +35,7 @@ LIBRARIES: Dict[str, str] = {
     "recurrence": "recurrence.hip",
     "linear_attention": "linear_attention.hip",
     "attn_capped": "attn_capped.hip",
+    "attn_capped_mfma": "attn_capped_mfma.hip",
     "moe": "moe.hip",
     "sampling": "sampling.hip",
     "probe": "probe.hip",

@@ -60,8 +60,12 @@ _PROTOTYPES = {
                            c_float, c_float, c_int, c_int, c_int, _P],
         "mf_rope_half_inplace": [_P, _P, _P, _P, c_int, c_int, c_int, c_int, c_int, _P],
     },
+    "attn_capped_mfma": {
+        "mf_capped_mfma": [_P, _P, _P, _P, c_int, _P, _P, _P, _P, c_int, _P, _P, c_int, c_int, c_int, c_int, c_float, c_float,
+                           c_int, _P],
+    },
     "moe": {
-        "mf_moe_route": [_P, _P, _P, _P, c_int, c_int, c_int, c_int, c_int, _P],
+        "mf_moe_route": [_P, c_int, _P, c_int, _P, _P, _P, c_int, c_int, c_int, c_int, c_int, _P],
         "mf_moe_act": [_P, _P, _P, c_int, c_int, c_int, c_int, c_float, _P],
         "mf_moe_sparse": [_P, _P, _P, _P, _P, _P, _P, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, _P],
     },
@@ -695,8 +699,6 @@ def qkv_conv_prep(qkv: torch.Tensor, conv_w: Optional[torch.Tensor], conv_state:
     for name, t, shape in (("cu_seqlens", cu_seqlens, (n_seqs + 1,)), ("seq_of_tok", seq_of_tok, (n_tok,)),
                            ("slot_ids", slot_ids, (n_seqs,)), ("positions", positions, (n_tok,))):
         _need(t, "qkv_conv_prep." + name, torch.int32, shape)
-    if C * 4 > 159 * 1024:
-        raise KernelError(f"qkv_conv_prep: rows of {C} channels do not fit into LDS")
     _check(_fn("attn_capped", "mf_qkv_conv_prep")(
         _ptr(qkv), _ptr(conv_w), taps, _ptr(conv_state if taps > 1 else None), _ptr(cu_seqlens), _ptr(seq_of_tok),
         _ptr(slot_ids), _ptr(positions), _ptr(cos), _ptr(sin), rot, float(blend), _ptr(v_first), _ptr(v_own),
@@ -735,10 +737,13 @@ def capped_attn(q: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tensor, pag
                           f"{v_dim} (at most 256)")
     if max_len > page_table.shape[1] * PAGE:
         raise KernelError(f"capped_attn: max_len {max_len} exceeds the page table ({page_table.shape[1]} pages)")
+    # keys split over workgroups where tokens x kv heads alone do not fill the chip: at least 256 keys a split;
+    # a windowed token's splits start at its window's first key
     reach = min(max_len, window) if window else max_len
-    n_splits, split_len = 1, max(PAGE, (max_len + PAGE - 1) // PAGE * PAGE)
-    if reach > 4 * PAGE and not (window and window < max_len):
-        n_splits, split_len = split_plan(n_tok, n_kv_heads, n_heads // n_kv_heads, 128, max_len)
+    blocks = n_tok * n_kv_heads * ((n_heads // n_kv_heads + 7) // 8)
+    n_splits = max(1, min(1024 // max(1, blocks), (reach + 255) // 256, 64))
+    split_len = ((reach + n_splits - 1) // n_splits + PAGE - 1) // PAGE * PAGE
+    n_splits = (reach + split_len - 1) // split_len
     part = workspace("attn", n_tok * n_heads * n_splits * (v_dim + 2), q.device) if n_splits > 1 else None
     _check(_fn("attn_capped", "mf_capped_attn")(
         _ptr(q), _ptr(kcache), _ptr(vcache), _ptr(page_table), page_table.shape[1], _ptr(positions), _ptr(seq_of_tok),
@@ -746,26 +751,66 @@ def capped_attn(q: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tensor, pag
         float(cap or 0.0), int(window or 0), n_splits, split_len, _stream()), "capped_attn")
 
 
+CAPPED_MFMA_ROWS = 16        # consecutive tokens of a sequence that a wave of the matrix-core form takes
+
+
+def capped_mfma_takes(dtype, dim: int, v_dim: int) -> bool:
+    """Whether the matrix-core form of the capped attention takes these sizes (it is compiled for them)."""
+    return dtype == torch.bfloat16 and dim % 16 == 0 and v_dim % 16 == 0 and 16 <= dim <= 256 and 16 <= v_dim <= 256
+
+
+def capped_attn_prefill(q: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tensor, page_table: torch.Tensor, ctx,
+                        temp: torch.Tensor, out: torch.Tensor, n_heads: int, n_kv_heads: int, dim: int, v_dim: int,
+                        scale: float, cap: float, window: int) -> None:
+    """`capped_attn` for a step with prompts or portions, bfloat16, on the matrix cores: blocks of 16
+    consecutive new tokens of a sequence (`ctx.query_tiles`) times the query heads of a kv head."""
+    n_tok = ctx.n_tokens
+    if not capped_mfma_takes(q.dtype, dim, v_dim):
+        raise KernelError(f"capped_attn_prefill: bfloat16 with keys and values of multiples of 16 up to 256; got "
+                          f"{q.dtype}, {dim}, {v_dim}")
+    _need(q, "capped_attn_prefill.q", torch.bfloat16, (n_tok, n_heads * dim))
+    _need(out, "capped_attn_prefill.out", torch.bfloat16, (n_tok, n_heads * v_dim))
+    _need_kv_pages("capped_attn_prefill", kcache, vcache, q.dtype, n_kv_heads, dim, v_dim)
+    _need(page_table, "capped_attn_prefill.page_table", torch.int32)
+    _need(temp, "capped_attn_prefill.temp", torch.float32, (n_heads,))
+    _need(ctx.cu_seqlens, "capped_attn_prefill.cu_seqlens", torch.int32, (ctx.n_seqs + 1,))
+    _need(ctx.start_pos, "capped_attn_prefill.start_pos", torch.int32, (ctx.n_seqs,))
+    if n_heads % n_kv_heads:
+        raise KernelError(f"capped_attn_prefill: {n_heads} heads over {n_kv_heads} kv heads")
+    if ctx.max_len > page_table.shape[1] * PAGE:
+        raise KernelError(f"capped_attn_prefill: max_len {ctx.max_len} exceeds the page table")
+    tile_seq, tile_q0 = ctx.query_tiles(CAPPED_MFMA_ROWS)
+    lib = build.variant("attn_capped_mfma", MF_CAPM_D=dim, MF_CAPM_V=v_dim)
+    _check(_fn("attn_capped_mfma", "mf_capped_mfma", lib)(
+        _ptr(q), _ptr(kcache), _ptr(vcache), _ptr(page_table), page_table.shape[1], _ptr(ctx.cu_seqlens),
+        _ptr(ctx.start_pos), _ptr(tile_seq), _ptr(tile_q0), tile_seq.numel(), _ptr(temp), _ptr(out), n_heads, n_kv_heads,
+        dim, v_dim, float(scale), float(cap or 0.0), int(window or 0), _stream()), "capped_attn_prefill")
+
+
 # ------------------------------------------------------------------ mixture of experts
 MOE_MAX_EXPERTS = 1024
+MOE_SPARSE_TOKENS, MOE_SPARSE_PAIRS = 16, 128     # what `moe_sparse` takes in one step (csrc/moe.hip)
 
 
-def moe_route(logits: torch.Tensor, dense: torch.Tensor, chosen: torch.Tensor, weights: torch.Tensor,
+def moe_route(x: torch.Tensor, router: torch.Tensor, dense: torch.Tensor, chosen: torch.Tensor, weights: torch.Tensor,
               n_groups: int, keep: int) -> None:
-    """From the router's 32-bit logits `[tokens][experts]`: softmax scores, the `keep` best of `n_groups`
-    groups of neighbouring experts (a group's score is its best expert's), the `chosen.shape[1]` best
-    experts of those groups, weighted by their scores over their sum.  `dense` `[tokens][experts]` gets the
-    weights at the chosen experts and 0 elsewhere; `chosen`, `weights` `[tokens][top]`."""
-    n_tok, E = logits.shape
+    """The router: logits = router x in 32-bit (`router` float32 `[experts][K]`, `x` `[tokens][K]` in the run
+    type), softmax scores, the `keep` best of `n_groups` groups of neighbouring experts (a group's score is
+    its best expert's), the `chosen.shape[1]` best experts of those groups, weighted by their scores over
+    their sum.  `dense` `[tokens][experts]` gets the weights at the chosen experts and 0 elsewhere; `chosen`,
+    `weights` `[tokens][top]`."""
+    n_tok, K = x.shape
+    E = router.shape[0]
     top = chosen.shape[1]
-    _need(logits, "moe_route.logits", torch.float32)
+    _need(x, "moe_route.x", _FLOATS)
+    _need(router, "moe_route.router", torch.float32, (E, K))
     _need(dense, "moe_route.dense", torch.float32, (n_tok, E))
     _need(chosen, "moe_route.chosen", torch.int32, (n_tok, top))
     _need(weights, "moe_route.weights", torch.float32, (n_tok, top))
     if E > MOE_MAX_EXPERTS or E % n_groups or not 1 <= keep <= n_groups or not 1 <= top <= min(64, keep * (E // n_groups)):
         raise KernelError(f"moe_route: {E} experts in {n_groups} groups, {keep} kept, {top} chosen")
-    _check(_fn("moe", "mf_moe_route")(_ptr(logits), _ptr(dense), _ptr(chosen), _ptr(weights), n_tok, E, n_groups, keep,
-                                       top, _stream()), "moe_route")
+    _check(_fn("moe", "mf_moe_route")(_ptr(x), _is_bf16(x), _ptr(router), K, _ptr(dense), _ptr(chosen), _ptr(weights),
+                                       n_tok, E, n_groups, keep, top, _stream()), "moe_route")
 
 
 def moe_act(gu: torch.Tensor, dense: torch.Tensor, out: torch.Tensor, limit: float) -> None:
@@ -797,6 +842,9 @@ def moe_sparse(x: torch.Tensor, gate_up: torch.Tensor, down: torch.Tensor, chose
     _need(chosen, "moe_sparse.chosen", torch.int32, (n_tok, top))
     _need(weights, "moe_sparse.weights", torch.float32, (n_tok, top))
     _need(out, "moe_sparse.out", torch.float32, (n_tok, N))
+    if n_tok > MOE_SPARSE_TOKENS or n_tok * top > MOE_SPARSE_PAIRS:
+        raise KernelError(f"moe_sparse: {n_tok} tokens with {top} experts each; it takes {MOE_SPARSE_TOKENS} tokens and "
+                          f"{MOE_SPARSE_PAIRS} pairs")
     y = torch.empty((n_tok, top, F), dtype=x.dtype, device=x.device)
     _check(_fn("moe", "mf_moe_sparse")(_ptr(x), _ptr(gate_up), _ptr(down), _ptr(chosen), _ptr(weights), _ptr(y), _ptr(out),
                                         _is_bf16(x), n_tok, top, n_experts, F, K, N, float(limit), _stream()), "moe_sparse")

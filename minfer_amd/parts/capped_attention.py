@@ -119,6 +119,11 @@ class CappedAttention(Mixer):
                           ctx.seq_of_tok, ctx.slot_ids, ctx.positions, cos, sin, self.blend, v_first, v_own, table,
                           q, kc, vc, self.nh, self.nk, self.dim, self.vdim, writes_cache)
         o = torch.empty((n, self.nh * self.vdim), dtype=self.rt.dtype, device=dev)
-        ops.capped_attn(q, kc, vc, table, ctx.positions, ctx.seq_of_tok, self.temp, o, self.nh, self.nk, self.dim,
-                        self.vdim, self.scale, self.cap, 0 if self.window is None else int(self.window), ctx.max_len)
+        window = 0 if self.window is None else int(self.window)
+        if not ctx.all_decode and ops.capped_mfma_takes(self.rt.dtype, self.dim, self.vdim):
+            ops.capped_attn_prefill(q, kc, vc, table, ctx, self.temp, o, self.nh, self.nk, self.dim, self.vdim, self.scale,
+                                    self.cap, window)
+        else:
+            ops.capped_attn(q, kc, vc, table, ctx.positions, ctx.seq_of_tok, self.temp, o, self.nh, self.nk, self.dim,
+                            self.vdim, self.scale, self.cap, window, ctx.max_len)
         self.o(o, out=h, accumulate=accumulate)

@@ -25,7 +25,7 @@ from .base import FeedForward, register_feed_forward
 from .linear import Linear
 
 # steps of at most this many tokens read only the chosen experts' matrices
-SPARSE_UP_TO = 16
+SPARSE_UP_TO = ops.MOE_SPARSE_TOKENS
 
 
 @register_feed_forward("grouped_moe")
@@ -59,7 +59,7 @@ class GroupedMoE(FeedForward):
         return s
 
     def load(self, get):
-        self.router = Linear(get(self.router_name).to(torch.float32))        # the router's product is 32-bit
+        self.router = get(self.router_name).to(torch.float32).contiguous()   # the router's product is 32-bit
         stems = [self.expert_name.format(e) for e in range(self.ne)]
         rows = []
         for s in stems:
@@ -72,15 +72,14 @@ class GroupedMoE(FeedForward):
 
     def forward(self, x, h, ctx, accumulate: bool = True) -> None:
         n, dev = x.shape[0], x.device
-        z = self.router(x, out_dtype=torch.float32)
         dense = torch.empty((n, self.ne), dtype=torch.float32, device=dev)
         chosen = torch.empty((n, self.top), dtype=torch.int32, device=dev)
         weights = torch.empty((n, self.top), dtype=torch.float32, device=dev)
-        ops.moe_route(z, dense, chosen, weights, self.groups, self.keep)
+        ops.moe_route(x, self.router, dense, chosen, weights, self.groups, self.keep)
         log = ctx._memo.get("route_log") if ctx is not None else None
         if log is not None:                  # a caller that wants to know: every routed layer's choices, in run order
             log.append(chosen)
-        if n <= SPARSE_UP_TO and x.dtype == self.gate_up.weight.dtype:
+        if n <= SPARSE_UP_TO and n * self.top <= ops.MOE_SPARSE_PAIRS and x.dtype == self.gate_up.weight.dtype:
             if not accumulate:
                 h.zero_()
             ops.moe_sparse(x, self.gate_up.weight, self.down.weight, chosen, weights, h, self.ne, self.limit)

@@ -470,11 +470,22 @@ def capped_attn(q, kcache, vcache, page_table, positions, seq_of_tok, temp, out,
             out[i, h * v_dim:(h + 1) * v_dim] = (torch.softmax(s, dim=0) @ vals).to(out.dtype)
 
 
+def capped_mfma_takes(dtype, dim, v_dim):
+    return dtype == torch.bfloat16 and dim % 16 == 0 and v_dim % 16 == 0 and 16 <= dim <= 256 and 16 <= v_dim <= 256
+
+
+def capped_attn_prefill(q, kcache, vcache, page_table, ctx, temp, out, n_heads, n_kv_heads, dim, v_dim, scale, cap, window):
+    capped_attn(q, kcache, vcache, page_table, ctx.positions, ctx.seq_of_tok, temp, out, n_heads, n_kv_heads, dim, v_dim,
+                scale, cap, window, ctx.max_len)
+
+
 # ------------------------------------------------------------------ mixture of experts
 MOE_MAX_EXPERTS = 1024
+MOE_SPARSE_TOKENS, MOE_SPARSE_PAIRS = 16, 128
 
 
-def moe_route(logits, dense, chosen, weights, n_groups, keep):
+def moe_route(x, router, dense, chosen, weights, n_groups, keep):
+    logits = (x.double() @ router.double().t()).float()
     n_tok, E = logits.shape
     top = chosen.shape[1]
     per = E // n_groups
@@ -593,7 +604,7 @@ NAMES = ["embed", "rmsnorm", "gather_rows", "swiglu", "convert", "fill_normal", 
          "group_rmsnorm", "xielu", "rope_table_freqs", "rope_pairs_inplace", "mingru_scan", "latent_prep",
          "headwise_linear", "latent_attn", "headwise_mfma_takes", "headwise_linear_mfma",
          "embed_pos", "gelu_tanh", "weighted_sum", "lightning_scan", "gated_rmsnorm", "rope_half_inplace",
-         "qkv_conv_prep", "capped_attn", "moe_route", "moe_act", "moe_sparse"]
+         "qkv_conv_prep", "capped_attn", "capped_mfma_takes", "capped_attn_prefill", "moe_route", "moe_act", "moe_sparse"]
 
 
 def install(monkeypatch):

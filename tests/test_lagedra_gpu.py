@@ -287,16 +287,63 @@ def test_a_key_at_the_window_edge_decides_or_is_not_seen(dtype, window, back, in
             assert row[2:].abs().max() < 10.0, (lens, new)
 
 
+def _step_context(lens, new, table, pos, seq):
+    from minfer_amd.engine.batch import StepContext
+    n = sum(new)
+    i32 = lambda v: torch.tensor(v, dtype=torch.int32, device=DEV)
+    return StepContext(cache=None, n_tokens=n, n_seqs=len(lens), token_ids=i32([0] * n), positions=pos.to(DEV),
+                       seq_of_tok=seq.to(DEV), cu_seqlens=i32(np.concatenate([[0], np.cumsum(new)]).tolist()),
+                       start_pos=i32([l - m for l, m in zip(lens, new)]), slot_ids=i32(list(range(len(lens)))),
+                       logit_rows=None, page_tables={}, max_len=max(lens), max_new=max(new), all_decode=False,
+                       host_new=list(new), host_start=[l - m for l, m in zip(lens, new)])
+
+
+@pytest.mark.parametrize("H, G, D, V, window, cap", [(6, 3, 32, 48, 17, 8.0), (8, 2, 96, 48, 40, 30.0), (4, 4, 16, 16, 0, 0.0),
+                                                     (16, 2, 128, 64, 70, 50.0), (7, 7, 48, 16, 1, 0.0), (2, 1, 64, 128, 33, 2.0)])
+@pytest.mark.parametrize("new", [(1, 130, 3, 1, 40), (1, 64, 64, 300, 65), (1, 1, 1, 2, 17)])
+def test_capped_attention_matrix_core_kernel(H, G, D, V, window, cap, new):
+    """The form for prompts and portions against the plain one: whole prompts, portions on held tokens and
+    single tokens in one launch, blocks of 16 tokens that end inside a sequence, over shuffled pages of a
+    poisoned pool."""
+    from minfer_amd.kernels import ops
+    lens = (1, 130, 64, 300, 65)
+    q, kc, vc, table, pos, seq, temp = _attention_case(torch.bfloat16, H, G, D, V, lens, new, window, cap, 4)
+    want = torch.empty(sum(new), H * V, dtype=torch.bfloat16)
+    plain_ops.capped_attn(q, kc, vc, table, pos, seq, temp, want, H, G, D, V, 0.2, cap, window, max(lens))
+    got = torch.empty(sum(new), H * V, dtype=torch.bfloat16, device=DEV)
+    ctx = _step_context(lens, new, table, pos, seq)
+    ops.capped_attn_prefill(q.to(DEV), kc.to(DEV), vc.to(DEV), table.to(DEV), ctx, temp.to(DEV), got, H, G, D, V, 0.2, cap,
+                            window)
+    err = (got.cpu().float() - want.float()).abs().max()
+    assert torch.isfinite(got).all() and err < 4e-2, float(err)
+
+
+@pytest.mark.parametrize("window, back, inside", [(17, 16, True), (17, 17, False), (70, 69, True), (70, 70, False),
+                                                  (0, 299, True), (65, 64, True), (64, 64, False), (33, 32, True), (32, 32, False)])
+def test_matrix_core_form_a_key_at_the_window_edge(window, back, inside):
+    from minfer_amd.kernels import ops
+    H, G, D, V = 4, 2, 16, 16
+    lens, new = (300, 90), (300, 20)
+    q, kc, vc, table, pos, seq, temp = _attention_case(torch.bfloat16, H, G, D, V, lens, new, window, 0.0, 5,
+                                                       needle=(0, 299 - back, 1))
+    got = torch.empty(sum(new), H * V, dtype=torch.bfloat16, device=DEV)
+    ops.capped_attn_prefill(q.to(DEV), kc.to(DEV), vc.to(DEV), table.to(DEV), _step_context(lens, new, table, pos, seq),
+                            temp.to(DEV), got, H, G, D, V, 1.0, 0.0, window)
+    row = got[new[0] - 1].float().cpu().view(H, V)
+    assert ((row[2:] - 50.0).abs().max() < 0.5) if inside else (row[2:].abs().max() < 10.0)
+
+
 def test_router_and_experts_kernels():
     from minfer_amd.kernels import ops
     for E, groups, keep, top, n in ((6, 3, 2, 3, 40), (8, 4, 4, 8, 5), (4, 1, 1, 1, 3), (64, 8, 3, 6, 33), (5, 5, 2, 2, 1)):
-        z = rnd(n, E, seed=E, scale=2.0)
         want = [torch.empty(n, E), torch.empty(n, top, dtype=torch.int32), torch.empty(n, top)]
         got = [t.clone().to(DEV) for t in want]
-        plain_ops.moe_route(z, want[0], want[1], want[2], groups, keep)
-        ops.moe_route(z.to(DEV), got[0], got[1], got[2], groups, keep)
-        assert torch.equal(got[1].cpu(), want[1]) and (got[0].cpu() - want[0]).abs().max() < 1e-6
-        assert (got[2].cpu() - want[2]).abs().max() < 1e-6
+        for xt in (torch.float32, torch.bfloat16):
+            xr, wr = rnd(n, 70, seed=E).to(xt), rnd(E, 70, seed=E + 1, scale=0.3)
+            plain_ops.moe_route(xr, wr, want[0], want[1], want[2], groups, keep)
+            ops.moe_route(xr.to(DEV), wr.to(DEV), got[0], got[1], got[2], groups, keep)
+            assert torch.equal(got[1].cpu(), want[1]) and (got[0].cpu() - want[0]).abs().max() < 1e-5
+            assert (got[2].cpu() - want[2]).abs().max() < 1e-5
         F, K, N = 24, 72, 40
         gu = rnd(n, E * 2 * F, seed=2, scale=2.0)
         for dtype, tol in ((torch.float32, 1e-5), (torch.bfloat16, 3e-2)):
@@ -306,9 +353,11 @@ def test_router_and_experts_kernels():
             assert (y.cpu().float() - y_want.float()).abs().max() < tol
             x, w1, w2 = rnd(n, K, seed=3).to(dtype), (rnd(E * 2 * F, K, seed=4) / 8).to(dtype), (rnd(N, E * F, seed=5) / 5).to(dtype)
             o_want, o = rnd(n, N, seed=6), rnd(n, N, seed=6).to(DEV)
-            plain_ops.moe_sparse(x, w1, w2, want[1], want[2], o_want, E, 1.5)
-            ops.moe_sparse(x.to(DEV), w1.to(DEV), w2.to(DEV), got[1], got[2], o, E, 1.5)
-            assert (o.cpu() - o_want).abs().max() < (1e-4 if dtype == torch.float32 else 5e-2)
+            few = min(n, 16)             # the step sizes the sparse form takes
+            plain_ops.moe_sparse(x[:few], w1, w2, want[1][:few], want[2][:few], o_want[:few], E, 1.5)
+            ops.moe_sparse(x[:few].contiguous().to(DEV), w1.to(DEV), w2.to(DEV), got[1][:few].contiguous(),
+                           got[2][:few].contiguous(), o[:few], E, 1.5)
+            assert (o.cpu()[:few] - o_want[:few]).abs().max() < (1e-4 if dtype == torch.float32 else 5e-2)
 
 
 def test_half_rotation_tables_and_kernel():
