@@ -3,8 +3,9 @@
 // compile time: the library is built for a model's sizes).  Semantics as `capped_attn_kernel`:
 // s = cap tanh(q . k scale temp[h] / cap), keys j with 0 <= p - j < window, softmax, o = sum p_j v_j.
 //
-// A wave owns 16 consecutive new tokens of one sequence times RB query heads of one kv head and walks the
-// tokens' keys 32 at a time (half a page), with no LDS and no barrier:
+// A wave (a workgroup of its own) owns 16 consecutive new tokens of one sequence times RB query heads of one kv
+// head and walks the tokens' keys 32 at a time (half a page), with no LDS and no barrier; the key rows of a
+// step are asked for a step ahead, the value rows before the step's scores are formed:
 //   S^T[key][token] = K Q^T      16x16x32 MFMA, A = 16 key rows straight from the cache, B = Q kept in registers
 //   a lane holds, for its token (lane % 16), the scores of keys 4 (lane / 16) + i of both key tiles:
 //   the softmax statistics are per lane, shared by the four lanes of a token through two shuffles
@@ -39,13 +40,13 @@ __device__ __forceinline__ float fast_tanh(float y) {
 }
 
 template <int RB>
-__global__ __launch_bounds__(256) void capped_mfma_kernel(
+__global__ __launch_bounds__(64) void capped_mfma_kernel(
     const bf16* __restrict__ q, const bf16* __restrict__ kc, const bf16* __restrict__ vc,
     const int* __restrict__ page_table, int pt_stride, const int* __restrict__ cu_seqlens,
     const int* __restrict__ start_pos, const int* __restrict__ tile_seq, const int* __restrict__ tile_q0, int n_tiles,
     const float* __restrict__ temp, bf16* __restrict__ out, int nh, int nk, float scale, float cap, int window) {
-  const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
-  const int tile = blockIdx.x * 4 + w;
+  const int lane = threadIdx.x & 63;
+  const int tile = blockIdx.x;                    // a workgroup is one wave: the waves drift apart freely
   if (tile >= n_tiles) return;
   const int G = nh / nk;
   const int n_hc = G / RB;
@@ -91,20 +92,40 @@ __global__ __launch_bounds__(256) void capped_mfma_kernel(
     for (int c = 0; c < NVT; ++c) oacc[r][c] = floatx4{0.f, 0.f, 0.f, 0.f};
   }
 
-  for (int kb = lo & ~31; kb <= p_last; kb += 32) {
+  // K fragments of both key tiles of the 32 keys from kb: key row `col` (+ 16), values 32 ks + 8 g .. + 8;
+  // they are asked for one step ahead
+  bf16x8 kn[2][DKS];
+  auto ask_k = [&](int kb) {
     const int page = pt[kb / MF_PAGE];
-    const int in_page = kb % MF_PAGE;              // 0 or 32
-    // K fragments of both key tiles: key row `col` (+ 16), values 32 ks + 8 g .. + 8
-    const bf16* kbase = kc + (((size_t)page * nk + hk) * MF_PAGE + in_page + col) * D + g * 8;
-    bf16x8 kf[2][DKS];
+    const bf16* kbase = kc + (((size_t)page * nk + hk) * MF_PAGE + kb % MF_PAGE + col) * D + g * 8;
 #pragma unroll
     for (int a = 0; a < 2; ++a)
 #pragma unroll
       for (int ks = 0; ks < DKS; ++ks) {
         bf16x8 v = {};
         if (ks * 32 + g * 8 < D) v = *(const bf16x8*)(kbase + (size_t)a * 16 * D + ks * 32);
-        kf[a][ks] = v;
+        kn[a][ks] = v;
       }
+  };
+  if ((lo & ~31) <= p_last) ask_k(lo & ~31);
+  for (int kb = lo & ~31; kb <= p_last; kb += 32) {
+    const int page = pt[kb / MF_PAGE];
+    const int in_page = kb % MF_PAGE;              // 0 or 32
+    bf16x8 kf[2][DKS];
+#pragma unroll
+    for (int a = 0; a < 2; ++a)
+#pragma unroll
+      for (int ks = 0; ks < DKS; ++ks) kf[a][ks] = kn[a][ks];
+    if (kb + 32 <= p_last) ask_k(kb + 32);
+    // V^T fragments: value row 16 c + col, keys 4 g .. + 4 and 16 + 4 g .. + 4 of this half page, asked for
+    // before the scores are formed
+    const bf16* vbase = vc + ((((size_t)page * nk + hk) * 2 + in_page / 32) * V + col) * 32 + 4 * g;
+    short4v vlo[NVT], vhi[NVT];
+#pragma unroll
+    for (int c = 0; c < NVT; ++c) {
+      vlo[c] = *(const short4v*)(vbase + (size_t)c * 16 * 32);
+      vhi[c] = *(const short4v*)(vbase + (size_t)c * 16 * 32 + 16);
+    }
     // which of this lane's 8 keys its token sees: slot j < 4: key kb + 4 g + j, else kb + 16 + 4 g + j - 4
     bool seen[8];
 #pragma unroll
@@ -148,13 +169,10 @@ __global__ __launch_bounds__(256) void capped_mfma_kernel(
 #pragma unroll
       for (int c = 0; c < NVT; ++c) oacc[r][c] *= corr;
     }
-    // V^T fragments: value row 16 c + col, keys 4 g .. + 4 and 16 + 4 g .. + 4 of this half page
-    const bf16* vbase = vc + ((((size_t)page * nk + hk) * 2 + in_page / 32) * V + col) * 32 + 4 * g;
     const bool tail = kb + 32 > seq_end;           // some of these keys were never written
 #pragma unroll
     for (int c = 0; c < NVT; ++c) {
-      const bf16* vp = vbase + (size_t)c * 16 * 32;
-      short4v lo4 = *(const short4v*)vp, hi4 = *(const short4v*)(vp + 16);
+      short4v lo4 = vlo[c], hi4 = vhi[c];
       if (tail) {
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
@@ -206,10 +224,12 @@ MF_API int mf_capped_mfma(const void* q, const void* kc, const void* vc, const i
   if (n_tiles <= 0) return 0;
   if (d != D || v != V || nk <= 0 || nh % nk || !temp) return (int)hipErrorInvalidValue;
   const int G = nh / nk;
-  const int rb = G % 4 == 0 ? 4 : (G % 2 == 0 ? 2 : 1);
-  dim3 grid((n_tiles + 3) / 4, nk * (G / rb));
+  // heads of a kv head a wave takes together: four where that still leaves waves for all SIMDs
+  int rb = G % 2 == 0 ? 2 : 1;
+  if (G % 4 == 0 && (long long)n_tiles * nk * (G / 4) >= 4096) rb = 4;
+  dim3 grid(n_tiles, nk * (G / rb));
 #define MF_GO(RB)                                                                                                          \
-  capped_mfma_kernel<RB><<<grid, 256, 0, stream>>>((const bf16*)q, (const bf16*)kc, (const bf16*)vc, page_table, pt_stride, \
+  capped_mfma_kernel<RB><<<grid, 64, 0, stream>>>((const bf16*)q, (const bf16*)kc, (const bf16*)vc, page_table, pt_stride, \
                                                    cu_seqlens, start_pos, tile_seq, tile_q0, n_tiles, temp, (bf16*)out, nh, \
                                                    nk, scale, cap, window)
   if (rb == 4) MF_GO(4);

@@ -91,42 +91,88 @@ __global__ __launch_bounds__(256) void lightning_scan_kernel(const float* __rest
 }
 
 // ------------------------------------------------------------------ the chunked form
-// chunk table: int32 [5][n_chunks] = first token, tokens, sequence, first chunk of the sequence, last or not
+// chunk table: int32 [2][n_chunks] = first token, tokens; then [n_seqs + 1] first chunks of the sequences
 //
-// pass 1: B_c[d][v] = sum_s decay^(n - 1 - s) k_s[d] v_s[v]; a workgroup owns (chunk, head, 64 columns),
-// threads as in the sequential kernel.
+// The products of the chunked form run on the matrix cores in 32-bit (16x16x4 MFMA with float operands: the
+// same multiply-adds as the plain form, no rounding of an operand): a lane gives A[i = lane % 16][k = lane / 16]
+// and B[k = lane / 16][j = lane % 16] and holds D[i = 4 (lane / 16) + r][j = lane % 16], r < 4.  Operands are
+// staged in LDS with rows 4 floats longer than they are, which spreads a fragment's 64 reads over the banks.
+#define MF_LA_VS (64 + 4)     // row stride of tiles of 64 columns
+
+// Staging of a [MF_LA_CHUNK][W] tile of 32-bit rows into LDS, silu applied or not: rows tt >= n and
+// columns beyond `valid` are zero.  With `vec` (every row start and `valid` multiples of 4 floats) a thread's
+// loads are 16 bytes each and all issued before the first is used.
+template <int WP, bool SILU>
+__device__ __forceinline__ void stage_tile(float* __restrict__ dst, int dst_stride, const float* __restrict__ src,
+                                           size_t src_stride, int n_rows, int n, int valid, bool vec) {
+  constexpr int W4 = WP / 4;
+  if (vec) {
+    for (int base = 0; base < n_rows * W4; base += 256 * 8) {
+      float4 tmp[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        const int i = base + u * 256 + threadIdx.x;
+        const int tt = i / W4, c4 = (i % W4) * 4;
+        tmp[u] = (i < n_rows * W4 && tt < n && c4 < valid) ? *(const float4*)(src + (size_t)tt * src_stride + c4)
+                                                             : float4{0.f, 0.f, 0.f, 0.f};
+      }
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        const int i = base + u * 256 + threadIdx.x;
+        if (i >= n_rows * W4) continue;
+        const int tt = i / W4, c4 = (i % W4) * 4;
+        float4 v = tmp[u];
+        if (SILU) { v.x = la_silu(v.x); v.y = la_silu(v.y); v.z = la_silu(v.z); v.w = la_silu(v.w); }
+        *(float4*)(dst + tt * dst_stride + c4) = v;
+      }
+    }
+  } else {
+    for (int i = threadIdx.x; i < n_rows * WP; i += 256) {
+      const int tt = i / WP, cc = i % WP;
+      const float v = (tt < n && cc < valid) ? src[(size_t)tt * src_stride + cc] : 0.f;
+      dst[tt * dst_stride + cc] = SILU ? la_silu(v) : v;
+    }
+  }
+}
+
+// pass 1: B_c[d][v] = sum_s decay^(n - 1 - s) k_s[d] v_s[v] = K'^T V; a workgroup owns (chunk, head, 64
+// columns), a wave 16 of the columns.
 template <int DS>
 __global__ __launch_bounds__(256) void lightning_chunk_sum_kernel(const float* __restrict__ proj, int row_len,
                                                                   const int* __restrict__ chunk_t0,
                                                                   const int* __restrict__ chunk_n,
                                                                   const float* __restrict__ decays,
                                                                   float* __restrict__ bsum, int H, int D, int V) {
-  __shared__ float sk[MF_LA_CHUNK][4 * DS + 1];
-  const int c = blockIdx.x, h = blockIdx.y;
-  const int col = blockIdx.z * 64 + (threadIdx.x & 63), slice = threadIdx.x >> 6;
-  const bool live = col < V;
+  constexpr int DP = 4 * DS, DPS = DP + 4;
+  extern __shared__ float lds[];
+  float* sk = lds;                          // [CHUNK][DPS]
+  float* sv = sk + MF_LA_CHUNK * DPS;       // [CHUNK][VS]
+  const int c = blockIdx.x, h = blockIdx.y, v0 = blockIdx.z * 64;
+  const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
   const int t0 = chunk_t0[c], n = chunk_n[c];
   const float decay = decays[h];
   const int off_k = H * D, off_v = 2 * H * D;
-  for (int i = threadIdx.x; i < n * 4 * DS; i += 256) {
-    const int tt = i / (4 * DS), d = i % (4 * DS);
-    sk[tt][d] = d < D ? la_silu(proj[(size_t)(t0 + tt) * row_len + off_k + h * D + d]) : 0.f;
-  }
+  const bool vec = D % 4 == 0 && V % 4 == 0;
+  const float* rows = proj + (size_t)t0 * row_len;
+  stage_tile<DP, true>(sk, DPS, rows + off_k + h * D, row_len, MF_LA_CHUNK, n, D, vec);
+  stage_tile<64, true>(sv, MF_LA_VS, rows + off_v + h * V + v0, row_len, MF_LA_CHUNK, n, min(64, V - v0), vec);
+  __shared__ float to_end[MF_LA_CHUNK];          // decay^(n - 1 - s): what a token's k v^T is worth at the chunk's end
+  if (threadIdx.x < MF_LA_CHUNK) to_end[threadIdx.x] = threadIdx.x < n ? powf(decay, (float)(n - 1 - threadIdx.x)) : 0.f;
   __syncthreads();
-  float B[DS];
+  const int col = lane & 15, g = lane >> 4;
+  for (int di = 0; di < DP / 16; ++di) {
+    floatx4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll 4
+    for (int kk = 0; kk < MF_LA_CHUNK / 4; ++kk) {
+      const int srow = 4 * kk + g;
+      acc = __builtin_amdgcn_mfma_f32_16x16x4f32(sk[srow * DPS + 16 * di + col] * to_end[srow], sv[srow * MF_LA_VS + 16 * w + col], acc,
+                                                 0, 0, 0);
+    }
+    const int cc = v0 + 16 * w + col;
 #pragma unroll
-  for (int i = 0; i < DS; ++i) B[i] = 0.f;
-  for (int tt = 0; tt < n; ++tt) {
-    const float vv = live ? la_silu(proj[(size_t)(t0 + tt) * row_len + off_v + h * V + col]) : 0.f;
-#pragma unroll
-    for (int i = 0; i < DS; ++i) B[i] = fmaf(decay, B[i], sk[tt][slice * DS + i] * vv);
-  }
-  if (live) {
-    float* b = bsum + (((size_t)c * H + h) * D) * V + col;
-#pragma unroll
-    for (int i = 0; i < DS; ++i) {
-      const int d = slice * DS + i;
-      if (d < D) b[(size_t)d * V] = B[i];
+    for (int r = 0; r < 4; ++r) {
+      const int dd = 16 * di + 4 * g + r;
+      if (dd < D && cc < V) bsum[(((size_t)c * H + h) * D + dd) * V + cc] = acc[r];
     }
   }
 }
@@ -156,10 +202,11 @@ __global__ __launch_bounds__(256) void lightning_chunk_fold_kernel(const int* __
   *st = S;
 }
 
-// pass 3: the outputs of a chunk from S_in and its own tokens.  A workgroup owns (chunk, head, 64
-// columns); q and k of the chunk are staged once, the decayed scores a[t][s] = decay^(t - s) (q_t . k_s),
-// s <= t, are formed by all threads, then thread (slice, column) adds the chunk's tokens for the output
-// rows t = slice, slice + 4, ...: o_t[v] = decay^(t + 1) sum_d q_t[d] S_in[d][v] + sum_s a[t][s] v_s[v].
+// pass 3: the outputs of a chunk from S_in and its own tokens.  A workgroup owns (chunk, head, 64 columns).
+// First the decayed scores a[t][s] = decay^(t - s) (q_t . k_s), s <= t, tile by tile (the tiles above the
+// diagonal are neither formed nor read), then for every 16 tokens x 16 columns
+// o = decay^(t + 1) (Q S_in) + a V: the first product's sums are scaled row by row before the second
+// product adds onto them.
 template <int DS>
 __global__ __launch_bounds__(256) void lightning_chunk_out_kernel(const float* __restrict__ proj, int row_len,
                                                                   const int* __restrict__ chunk_t0,
@@ -167,52 +214,64 @@ __global__ __launch_bounds__(256) void lightning_chunk_out_kernel(const float* _
                                                                   const float* __restrict__ decays,
                                                                   const float* __restrict__ s_in,
                                                                   float* __restrict__ out, int H, int D, int V) {
+  constexpr int DP = 4 * DS, DPS = DP + 4;
   extern __shared__ float lds[];
-  constexpr int DP = 4 * DS;
-  float* sq = lds;                                   // [CHUNK][DP + 1]
-  float* sk = sq + MF_LA_CHUNK * (DP + 1);            // [CHUNK][DP + 1]
-  float* sa = sk + MF_LA_CHUNK * (DP + 1);            // [CHUNK][CHUNK + 1]
-  float* sv = sa + MF_LA_CHUNK * (MF_LA_CHUNK + 1);   // [CHUNK][64]
-  float* ss = sv + MF_LA_CHUNK * 64;                  // [DP][64]: S_in of this head and these columns
-  const int c = blockIdx.x, h = blockIdx.y;
-  const int lane = threadIdx.x & 63, slice = threadIdx.x >> 6;
-  const int col = blockIdx.z * 64 + lane;
-  const bool live = col < V;
+  float* sq = lds;                                   // [CHUNK][DPS]
+  float* sk = sq + MF_LA_CHUNK * DPS;                 // [CHUNK][DPS]
+  float* sa = sk + MF_LA_CHUNK * DPS;                 // [CHUNK][VS]: decayed scores
+  float* sv = sa + MF_LA_CHUNK * MF_LA_VS;            // [CHUNK][VS]
+  float* ss = sv + MF_LA_CHUNK * MF_LA_VS;            // [DP][VS]: S_in of this head and these columns
+  float* dpow = ss + DP * MF_LA_VS;                   // [CHUNK + 1]: decay^i
+  const int c = blockIdx.x, h = blockIdx.y, v0 = blockIdx.z * 64;
+  const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
   const int t0 = chunk_t0[c], n = chunk_n[c];
   const float decay = decays[h];
   const int off_k = H * D, off_v = 2 * H * D;
-  for (int i = threadIdx.x; i < n * DP; i += 256) {
-    const int tt = i / DP, d = i % DP;
-    const float* row = proj + (size_t)(t0 + tt) * row_len + h * D + d;
-    sq[tt * (DP + 1) + d] = d < D ? la_silu(row[0]) : 0.f;
-    sk[tt * (DP + 1) + d] = d < D ? la_silu(row[off_k]) : 0.f;
-  }
-  for (int i = threadIdx.x; i < n * 64; i += 256) {
-    const int tt = i >> 6, cc = blockIdx.z * 64 + (i & 63);
-    sv[i] = cc < V ? la_silu(proj[(size_t)(t0 + tt) * row_len + off_v + h * V + cc]) : 0.f;
-  }
-  const float* sin_base = s_in + (((size_t)c * H + h) * D) * V;
-  for (int i = threadIdx.x; i < DP * 64; i += 256) {
-    const int d = i >> 6, cc = blockIdx.z * 64 + (i & 63);
-    ss[i] = (d < D && cc < V) ? sin_base[(size_t)d * V + cc] : 0.f;
-  }
+  const bool vec = D % 4 == 0 && V % 4 == 0;
+  const float* rows = proj + (size_t)t0 * row_len;
+  stage_tile<DP, true>(sq, DPS, rows + h * D, row_len, MF_LA_CHUNK, n, D, vec);
+  stage_tile<DP, true>(sk, DPS, rows + off_k + h * D, row_len, MF_LA_CHUNK, n, D, vec);
+  stage_tile<64, true>(sv, MF_LA_VS, rows + off_v + h * V + v0, row_len, MF_LA_CHUNK, n, min(64, V - v0), vec);
+  stage_tile<64, false>(ss, MF_LA_VS, s_in + (((size_t)c * H + h) * D) * V + v0, V, DP, D, min(64, V - v0), vec);
+  if (threadIdx.x <= MF_LA_CHUNK) dpow[threadIdx.x] = powf(decay, (float)threadIdx.x);
   __syncthreads();
-  for (int i = threadIdx.x; i < n * n; i += 256) {
-    const int t = i / n, s = i % n;
-    float a = 0.f;
-    if (s <= t) {
-      for (int d = 0; d < DP; ++d) a = fmaf(sq[t * (DP + 1) + d], sk[s * (DP + 1) + d], a);
-      a *= powf(decay, (float)(t - s));
+  const int col = lane & 15, g = lane >> 4;
+  // the ten score tiles on and below the diagonal, in turn over the waves
+  for (int tile = w; tile < 10; tile += 4) {
+    int ti = 0, rest = tile;
+    while (rest > ti) { rest -= ti + 1; ++ti; }       // tile -> (ti, sj = rest), sj <= ti
+    const int sj = rest;
+    floatx4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll 4
+    for (int kk = 0; kk < DP / 4; ++kk)
+      acc = __builtin_amdgcn_mfma_f32_16x16x4f32(sq[(16 * ti + col) * DPS + 4 * kk + g], sk[(16 * sj + col) * DPS + 4 * kk + g],
+                                                 acc, 0, 0, 0);
+    const int sidx = 16 * sj + col;
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const int t = 16 * ti + 4 * g + r;
+      sa[t * MF_LA_VS + sidx] = sidx <= t ? acc[r] * dpow[t - sidx] : 0.f;
     }
-    sa[t * (MF_LA_CHUNK + 1) + s] = a;
   }
   __syncthreads();
-  for (int t = slice; t < n; t += 4) {
-    float cross = 0.f;
-    for (int d = 0; d < DP; ++d) cross = fmaf(sq[t * (DP + 1) + d], ss[d * 64 + lane], cross);
-    float o = cross * powf(decay, (float)(t + 1));
-    for (int s = 0; s <= t; ++s) o = fmaf(sa[t * (MF_LA_CHUNK + 1) + s], sv[s * 64 + lane], o);
-    if (live) out[(size_t)(t0 + t) * H * V + h * V + col] = o;
+  const int cc = v0 + 16 * w + col;
+  for (int ti = 0; ti < MF_LA_CHUNK / 16 && 16 * ti < n; ++ti) {
+    floatx4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll 4
+    for (int kk = 0; kk < DP / 4; ++kk)
+      acc = __builtin_amdgcn_mfma_f32_16x16x4f32(sq[(16 * ti + col) * DPS + 4 * kk + g], ss[(4 * kk + g) * MF_LA_VS + 16 * w + col],
+                                                 acc, 0, 0, 0);
+#pragma unroll
+    for (int r = 0; r < 4; ++r) acc[r] *= dpow[16 * ti + 4 * g + r + 1];
+#pragma unroll 4
+    for (int kk = 0; kk < 4 * (ti + 1); ++kk)
+      acc = __builtin_amdgcn_mfma_f32_16x16x4f32(sa[(16 * ti + col) * MF_LA_VS + 4 * kk + g], sv[(4 * kk + g) * MF_LA_VS + 16 * w + col],
+                                                 acc, 0, 0, 0);
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const int t = 16 * ti + 4 * g + r;
+      if (t < n && cc < V) out[(size_t)(t0 + t) * H * V + h * V + cc] = acc[r];
+    }
   }
 }
 
@@ -261,15 +320,27 @@ MF_API int mf_lightning_scan_chunked(const float* proj, const int* chunks, int n
                                      const int* slot_ids, const float* decays, float* state, float* bsum, float* out,
                                      int n_seqs, int H, int D, int V, hipStream_t stream) {
   if (n_seqs <= 0 || n_chunks <= 0) return 0;
-  if (H <= 0 || D <= 0 || V <= 0 || D > 256 || !bsum) return (int)hipErrorInvalidValue;
+  if (H <= 0 || D <= 0 || V <= 0 || D > 128 || !bsum) return (int)hipErrorInvalidValue;
   const int row_len = 2 * H * D + 2 * H * V;
   const int* t0 = chunks;
   const int* n = chunks + n_chunks;
   dim3 grid(n_chunks, H, (V + 63) / 64);
-#define MF_CALL(DS) lightning_chunk_sum_kernel<DS><<<grid, 256, 0, stream>>>(proj, row_len, t0, n, decays, bsum, H, D, V);
+  int rc = 0;
+#define MF_CALL(DS)                                                                                                   \
+  {                                                                                                                   \
+    const size_t lds = sizeof(float) * (MF_LA_CHUNK * (4 * DS + 4) + MF_LA_CHUNK * MF_LA_VS);                         \
+    static bool raised = false;                                                                                       \
+    if (!raised && lds > 48 * 1024) {                                                                                 \
+      rc = (int)hipFuncSetAttribute((const void*)lightning_chunk_sum_kernel<DS>,                                      \
+                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);                            \
+      if (rc) return rc;                                                                                              \
+      raised = true;                                                                                                  \
+    }                                                                                                                 \
+    lightning_chunk_sum_kernel<DS><<<grid, 256, lds, stream>>>(proj, row_len, t0, n, decays, bsum, H, D, V);          \
+  }
   MF_LA_DISPATCH(MF_CALL)
 #undef MF_CALL
-  int rc = mf_launch_status();
+  rc = mf_launch_status();
   if (rc) return rc;
   lightning_chunk_fold_kernel<<<dim3(n_seqs, H, (D * V + 255) / 256), 256, 0, stream>>>(n, seq_first_chunk, slot_ids, decays,
                                                                                         bsum, state, H, D * V);
@@ -277,8 +348,8 @@ MF_API int mf_lightning_scan_chunked(const float* proj, const int* chunks, int n
   if (rc) return rc;
 #define MF_CALL(DS)                                                                                                   \
   {                                                                                                                   \
-    const size_t lds = sizeof(float) * (2 * MF_LA_CHUNK * (4 * DS + 1) + MF_LA_CHUNK * (MF_LA_CHUNK + 1) +            \
-                                        MF_LA_CHUNK * 64 + 4 * DS * 64);                                              \
+    const size_t lds = sizeof(float) * (2 * MF_LA_CHUNK * (4 * DS + 4) + 2 * MF_LA_CHUNK * MF_LA_VS +                 \
+                                        4 * DS * MF_LA_VS + MF_LA_CHUNK + 1);                                         \
     static bool raised = false;                                                                                       \
     if (!raised && lds > 48 * 1024) {                                                                                 \
       rc = (int)hipFuncSetAttribute((const void*)lightning_chunk_out_kernel<DS>,                                      \
