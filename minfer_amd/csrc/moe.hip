@@ -80,7 +80,10 @@ __global__ __launch_bounds__(256) void moe_route_kernel(const XT* __restrict__ x
   for (int e = lane; e < E; e += 64) { const float v = expf(s[e] - mx); s[e] = v; sum += v; }
   sum = wave_sum(sum);
   MF_WAVE_SYNC();
-  for (int e = lane; e < E; e += 64) { s[e] = s[e] / sum; dense[(size_t)t * E + e] = 0.f; }
+  for (int e = lane; e < E; e += 64) {
+    s[e] = s[e] / sum;
+    if (dense) dense[(size_t)t * E + e] = 0.f;
+  }
   MF_WAVE_SYNC();
   const int per = E / n_groups;
   for (int g = lane; g < n_groups; g += 64) {
@@ -117,7 +120,7 @@ __global__ __launch_bounds__(256) void moe_route_kernel(const XT* __restrict__ x
   }
   if (lane < top) {
     const float wgt = s[mine] / (wsum + 1e-20f);
-    dense[(size_t)t * E + mine] = wgt;
+    if (dense) dense[(size_t)t * E + mine] = wgt;
     chosen[(size_t)t * top + lane] = mine;
     weights[(size_t)t * top + lane] = wgt;
   }
@@ -225,8 +228,8 @@ __global__ __launch_bounds__(256) void moe_sparse_up_kernel(const WT* __restrict
   }
 }
 
-// down [N][E F] (the experts' down matrices side by side), y [tokens][top][F]:
-// out[t][n] += sum_k w[t][k] dot(down[n][e_k F .. e_k F + F), y[t][k]), a token's choices added in their order.
+// down [E][N][F], y [tokens][top][F]:
+// out[t][n] += sum_k w[t][k] dot(down[e_k][n], y[t][k]), a token's choices added in their order.
 // A wave owns output n: for every expert that has pairs, its part of row n is read once and meets the y rows
 // of the expert's pairs; lane p % 64 keeps pair p's dot product until the tokens' sums are formed.
 template <typename WT>
@@ -247,7 +250,7 @@ __global__ __launch_bounds__(256) void moe_sparse_down_kernel(const WT* __restri
     const unsigned long long before0 = i < 64 ? (i ? ~0ull >> (64 - i) : 0ull) : ~0ull;
     const unsigned long long before1 = i <= 64 ? 0ull : ~0ull >> (128 - i);
     if ((mine0 & before0) | (mine1 & before1)) continue;       // an earlier pair led this expert
-    const WT* wr = down + (size_t)n * E * F + (size_t)e * F;
+    const WT* wr = down + ((size_t)e * N + n) * F;
     float acc[MF_MOE_SPARSE_TOKENS];
 #pragma unroll
     for (int j = 0; j < MF_MOE_SPARSE_TOKENS; ++j) acc[j] = 0.f;
@@ -283,6 +286,59 @@ __global__ __launch_bounds__(256) void moe_sparse_down_kernel(const WT* __restri
     total = fmaf(weights[pr], pr < 64 ? d0 : d1, total);
   }
   if (lane < n_tok) out[(size_t)lane * N + n] += total;
+}
+
+// ------------------------------------------------------------------ many tokens: the tokens of an expert together
+// `moe_group_kernel`: a workgroup per expert walks the step's (token, choice) pairs in order and gives
+// every pair of its expert its rank among them; counts[e] is their number.  With the experts' offsets
+// (the running sum of the counts, formed by the host) pair p stands in row offsets[chosen[p]] + rank[p] of the
+// buffers that hold the experts' tokens one expert after the other.
+__global__ __launch_bounds__(256) void moe_group_kernel(const int* __restrict__ chosen, int n_pairs, int* __restrict__ rank,
+                                                        int* __restrict__ counts) {
+  __shared__ int wave_count[4];
+  const int e = blockIdx.x;
+  const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+  int before = 0;
+  for (int p0 = 0; p0 < n_pairs; p0 += 256) {
+    const int p = p0 + threadIdx.x;
+    const bool mine = p < n_pairs && chosen[p] == e;
+    const unsigned long long m = __ballot(mine);
+    __syncthreads();
+    if (lane == 0) wave_count[w] = __popcll(m);
+    __syncthreads();
+    int ahead = before;
+    for (int i = 0; i < w; ++i) ahead += wave_count[i];
+    if (mine) rank[p] = ahead + __popcll(m & ((1ull << lane) - 1));
+    before += wave_count[0] + wave_count[1] + wave_count[2] + wave_count[3];
+  }
+  if (threadIdx.x == 0) counts[e] = before;
+}
+
+// xs[row(p)][:] = x[p / top][:]
+template <typename T>
+__global__ __launch_bounds__(256) void moe_gather_kernel(const T* __restrict__ x, const int* __restrict__ chosen,
+                                                         const int* __restrict__ rank, const int* __restrict__ offsets,
+                                                         T* __restrict__ xs, int top, int K) {
+  const int p = blockIdx.x;
+  const T* src = x + (size_t)(p / top) * K;
+  T* dst = xs + (size_t)(offsets[chosen[p]] + rank[p]) * K;
+  for (int i = threadIdx.x; i < K; i += 256) dst[i] = src[i];
+}
+
+// out[t][:] (+)= sum_k w[t][k] rows[row(t top + k)][:], the choices in their order
+__global__ __launch_bounds__(256) void moe_combine_kernel(const float* __restrict__ rows, const int* __restrict__ chosen,
+                                                          const int* __restrict__ rank, const int* __restrict__ offsets,
+                                                          const float* __restrict__ weights, float* __restrict__ out,
+                                                          int top, int N, int add) {
+  const int t = blockIdx.x;
+  const int i = blockIdx.y * 256 + threadIdx.x;
+  if (i >= N) return;
+  float a = add ? out[(size_t)t * N + i] : 0.f;
+  for (int k = 0; k < top; ++k) {
+    const int p = t * top + k;
+    a = fmaf(weights[p], rows[(size_t)(offsets[chosen[p]] + rank[p]) * N + i], a);
+  }
+  out[(size_t)t * N + i] = a;
 }
 
 // ------------------------------------------------------------------ entry points
@@ -330,5 +386,28 @@ MF_API int mf_moe_sparse(const void* x, const void* gate_up, const void* down, c
     if (rc) return rc;
     moe_sparse_down_kernel<float><<<g2, 256, 0, stream>>>((const float*)y, (const float*)down, chosen, weights, out, n_tok, top, E, F, N);
   }
+  return mf_launch_status();
+}
+
+MF_API int mf_moe_group(const int* chosen, int n_pairs, int E, int* rank, int* counts, hipStream_t stream) {
+  if (n_pairs <= 0 || E <= 0) return 0;
+  moe_group_kernel<<<E, 256, 0, stream>>>(chosen, n_pairs, rank, counts);
+  return mf_launch_status();
+}
+
+MF_API int mf_moe_gather(const void* x, int is_bf16, const int* chosen, const int* rank, const int* offsets, void* xs,
+                         int n_pairs, int top, int K, hipStream_t stream) {
+  if (n_pairs <= 0) return 0;
+  if (is_bf16)
+    moe_gather_kernel<bf16><<<n_pairs, 256, 0, stream>>>((const bf16*)x, chosen, rank, offsets, (bf16*)xs, top, K);
+  else
+    moe_gather_kernel<float><<<n_pairs, 256, 0, stream>>>((const float*)x, chosen, rank, offsets, (float*)xs, top, K);
+  return mf_launch_status();
+}
+
+MF_API int mf_moe_combine(const float* rows, const int* chosen, const int* rank, const int* offsets, const float* weights,
+                          float* out, int n_tok, int top, int N, int add, hipStream_t stream) {
+  if (n_tok <= 0) return 0;
+  moe_combine_kernel<<<dim3(n_tok, (N + 255) / 256), 256, 0, stream>>>(rows, chosen, rank, offsets, weights, out, top, N, add);
   return mf_launch_status();
 }

@@ -68,6 +68,9 @@ _PROTOTYPES = {
         "mf_moe_route": [_P, c_int, _P, c_int, _P, _P, _P, c_int, c_int, c_int, c_int, c_int, _P],
         "mf_moe_act": [_P, _P, _P, c_int, c_int, c_int, c_int, c_float, _P],
         "mf_moe_sparse": [_P, _P, _P, _P, _P, _P, _P, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, _P],
+        "mf_moe_group": [_P, c_int, c_int, _P, _P, _P],
+        "mf_moe_gather": [_P, c_int, _P, _P, _P, _P, c_int, c_int, c_int, _P],
+        "mf_moe_combine": [_P, _P, _P, _P, _P, _P, c_int, c_int, c_int, c_int, _P],
     },
     "recurrence": {
         "mf_mingru_scan": [_P, _P, _P, _P, _P, c_int, c_int, c_int, _P],
@@ -792,19 +795,20 @@ MOE_MAX_EXPERTS = 1024
 MOE_SPARSE_TOKENS, MOE_SPARSE_PAIRS = 16, 128     # what `moe_sparse` takes in one step (csrc/moe.hip)
 
 
-def moe_route(x: torch.Tensor, router: torch.Tensor, dense: torch.Tensor, chosen: torch.Tensor, weights: torch.Tensor,
-              n_groups: int, keep: int) -> None:
+def moe_route(x: torch.Tensor, router: torch.Tensor, dense: Optional[torch.Tensor], chosen: torch.Tensor,
+              weights: torch.Tensor, n_groups: int, keep: int) -> None:
     """The router: logits = router x in 32-bit (`router` float32 `[experts][K]`, `x` `[tokens][K]` in the run
     type), softmax scores, the `keep` best of `n_groups` groups of neighbouring experts (a group's score is
     its best expert's), the `chosen.shape[1]` best experts of those groups, weighted by their scores over
-    their sum.  `dense` `[tokens][experts]` gets the weights at the chosen experts and 0 elsewhere; `chosen`,
-    `weights` `[tokens][top]`."""
+    their sum.  `dense` `[tokens][experts]`, where given, gets the weights at the chosen experts and 0
+    elsewhere; `chosen`, `weights` `[tokens][top]`."""
     n_tok, K = x.shape
     E = router.shape[0]
     top = chosen.shape[1]
     _need(x, "moe_route.x", _FLOATS)
     _need(router, "moe_route.router", torch.float32, (E, K))
-    _need(dense, "moe_route.dense", torch.float32, (n_tok, E))
+    if dense is not None:
+        _need(dense, "moe_route.dense", torch.float32, (n_tok, E))
     _need(chosen, "moe_route.chosen", torch.int32, (n_tok, top))
     _need(weights, "moe_route.weights", torch.float32, (n_tok, top))
     if E > MOE_MAX_EXPERTS or E % n_groups or not 1 <= keep <= n_groups or not 1 <= top <= min(64, keep * (E // n_groups)):
@@ -830,15 +834,14 @@ def moe_act(gu: torch.Tensor, dense: torch.Tensor, out: torch.Tensor, limit: flo
 def moe_sparse(x: torch.Tensor, gate_up: torch.Tensor, down: torch.Tensor, chosen: torch.Tensor, weights: torch.Tensor,
                out: torch.Tensor, n_experts: int, limit: float) -> None:
     """The chosen experts only, for steps of few tokens: `gate_up` `[experts][2 F][K]` (an expert's gate
-    rows, then its up rows), `down` `[N][experts F]`; out `[tokens][N]` float32 += the weighted sum of the
+    rows, then its up rows), `down` `[experts][N][F]`; out `[tokens][N]` float32 += the weighted sum of the
     chosen experts' outputs, choices added in their order."""
     n_tok, K = x.shape
     top = chosen.shape[1]
-    N, EF = down.shape
-    F = EF // n_experts
+    _, N, F = down.shape
     _need(x, "moe_sparse.x", _FLOATS)
-    _need(gate_up, "moe_sparse.gate_up", x.dtype, (2 * EF, K))
-    _need(down, "moe_sparse.down", x.dtype, (N, n_experts * F))
+    _need(gate_up, "moe_sparse.gate_up", x.dtype, (n_experts, 2 * F, K))
+    _need(down, "moe_sparse.down", x.dtype, (n_experts, N, F))
     _need(chosen, "moe_sparse.chosen", torch.int32, (n_tok, top))
     _need(weights, "moe_sparse.weights", torch.float32, (n_tok, top))
     _need(out, "moe_sparse.out", torch.float32, (n_tok, N))
@@ -1715,3 +1718,41 @@ def probe_mfma(rounds: int, blocks: Optional[int] = None, device="cuda") -> floa
     sink = workspace("probe", blocks, device)
     _check(_fn("probe", "mf_probe_mfma")(int(rounds), _ptr(sink), blocks, _stream()), "probe_mfma")
     return float(blocks) * 8 * rounds * 8 * 2 * 32 * 32 * 16
+
+
+def moe_group(chosen: torch.Tensor, n_experts: int, rank: torch.Tensor, counts: torch.Tensor) -> None:
+    """`rank[t][k]`: how many earlier (token, choice) pairs of the step chose the same expert; `counts[e]`:
+    the pairs of expert e."""
+    _need(chosen, "moe_group.chosen", torch.int32)
+    _need(rank, "moe_group.rank", torch.int32, tuple(chosen.shape))
+    _need(counts, "moe_group.counts", torch.int32, (n_experts,))
+    _check(_fn("moe", "mf_moe_group")(_ptr(chosen), chosen.numel(), n_experts, _ptr(rank), _ptr(counts), _stream()), "moe_group")
+
+
+def moe_gather(x: torch.Tensor, chosen: torch.Tensor, rank: torch.Tensor, offsets: torch.Tensor, xs: torch.Tensor) -> None:
+    """xs[offsets[chosen[t][k]] + rank[t][k]] = x[t]: the tokens of every expert side by side, one expert after
+    the other."""
+    n_tok, K = x.shape
+    top = chosen.shape[1]
+    _need(x, "moe_gather.x", _FLOATS)
+    _need(chosen, "moe_gather.chosen", torch.int32, (n_tok, top))
+    _need(rank, "moe_gather.rank", torch.int32, (n_tok, top))
+    _need(offsets, "moe_gather.offsets", torch.int32)
+    _need(xs, "moe_gather.xs", x.dtype, (n_tok * top, K))
+    _check(_fn("moe", "mf_moe_gather")(_ptr(x), _is_bf16(x), _ptr(chosen), _ptr(rank), _ptr(offsets), _ptr(xs), n_tok * top,
+                                        top, K, _stream()), "moe_gather")
+
+
+def moe_combine(rows: torch.Tensor, chosen: torch.Tensor, rank: torch.Tensor, offsets: torch.Tensor, weights: torch.Tensor,
+                out: torch.Tensor, accumulate: bool = True) -> None:
+    """out[t] (+)= sum_k weights[t][k] rows[offsets[chosen[t][k]] + rank[t][k]], a token's choices in their order."""
+    n_tok, top = chosen.shape
+    N = out.shape[1]
+    _need(rows, "moe_combine.rows", torch.float32, (n_tok * top, N))
+    _need(chosen, "moe_combine.chosen", torch.int32)
+    _need(rank, "moe_combine.rank", torch.int32, (n_tok, top))
+    _need(offsets, "moe_combine.offsets", torch.int32)
+    _need(weights, "moe_combine.weights", torch.float32, (n_tok, top))
+    _need(out, "moe_combine.out", torch.float32, (n_tok, N))
+    _check(_fn("moe", "mf_moe_combine")(_ptr(rows), _ptr(chosen), _ptr(rank), _ptr(offsets), _ptr(weights), _ptr(out), n_tok,
+                                         top, N, 1 if accumulate else 0, _stream()), "moe_combine")

@@ -6,11 +6,12 @@ can be among the `top` chosen; the chosen experts' scores over their sum are the
 Expert (no biases): g = min(Wg x, limit), u = clamp(Wu x, -limit, limit), y = g sigmoid(1.702 g) (u + 1),
 output Wd y.  The result is the weighted sum of the chosen experts' outputs.
 
-Two forms.  Steps of many tokens run every expert's gate|up over all tokens as one product (the
-experts' matrices stacked), apply the activation times the token's weight for the expert (0 where it
-was not chosen) and multiply by the experts' down matrices side by side: two products whatever
-the routing, experts / top times the arithmetic of the chosen experts alone.  Steps of few tokens
-read only the chosen experts' matrices (`ops.moe_sparse`).
+Two forms, both of which read or multiply only what was chosen.  Steps of few tokens and decode steps (which
+may be captured, so nothing may wait for the host): `ops.moe_sparse`, up to 16 tokens a launch, reads every
+chosen expert's matrices once.  Steps of many tokens: the (token, choice) pairs are grouped by expert
+(`ops.moe_group`; the host reads the experts' counts, the one wait of the step), the tokens' rows are put side by
+side expert by expert, every expert with tokens runs its two products over its rows, and the rows' results are
+added into the stream with the tokens' weights, a token's choices in their order.
 
 A step whose context carries a list under `_memo["route_log"]` gets every routed layer's choices
 (`[rows][top]` expert numbers, on the device) appended to it, in run order.
@@ -61,30 +62,58 @@ class GroupedMoE(FeedForward):
     def load(self, get):
         self.router = get(self.router_name).to(torch.float32).contiguous()   # the router's product is 32-bit
         stems = [self.expert_name.format(e) for e in range(self.ne)]
-        rows = []
-        for s in stems:
-            rows += [get(s + ".gate"), get(s + ".up")]
-        self.gate_up = Linear.stacked(rows)                                  # [experts][gate | up][hidden]
-        self.down = Linear(torch.cat([get(s + ".down") for s in stems], dim=1).contiguous())   # [hidden][experts x inter]
+        # [experts][gate | up][hidden] and [experts][hidden][inter]: an expert's matrices are contiguous slices
+        self.gate_up = torch.stack([torch.cat([get(s + ".gate"), get(s + ".up")], dim=0) for s in stems]).contiguous()
+        self.down = torch.stack([get(s + ".down") for s in stems]).contiguous()
+        self.experts = [(Linear(self.gate_up[e]), Linear(self.down[e])) for e in range(self.ne)]
 
     def decode_copies(self, make: bool, min_row_length: int = 0) -> int:
         return 0
 
     def forward(self, x, h, ctx, accumulate: bool = True) -> None:
         n, dev = x.shape[0], x.device
-        dense = torch.empty((n, self.ne), dtype=torch.float32, device=dev)
         chosen = torch.empty((n, self.top), dtype=torch.int32, device=dev)
         weights = torch.empty((n, self.top), dtype=torch.float32, device=dev)
-        ops.moe_route(x, self.router, dense, chosen, weights, self.groups, self.keep)
+        ops.moe_route(x, self.router, None, chosen, weights, self.groups, self.keep)
         log = ctx._memo.get("route_log") if ctx is not None else None
         if log is not None:                  # a caller that wants to know: every routed layer's choices, in run order
             log.append(chosen)
-        if n <= SPARSE_UP_TO and n * self.top <= ops.MOE_SPARSE_PAIRS and x.dtype == self.gate_up.weight.dtype:
+        if n == 0:
+            return
+        few = min(SPARSE_UP_TO, max(1, ops.MOE_SPARSE_PAIRS // self.top))
+        if (n <= few or (ctx is not None and ctx.all_decode)) and x.dtype == self.gate_up.dtype:
             if not accumulate:
                 h.zero_()
-            ops.moe_sparse(x, self.gate_up.weight, self.down.weight, chosen, weights, h, self.ne, self.limit)
+            for t0 in range(0, n, few):      # (slices of a contiguous tensor's rows are contiguous)
+                ops.moe_sparse(x[t0:t0 + few], self.gate_up, self.down, chosen[t0:t0 + few], weights[t0:t0 + few],
+                               h[t0:t0 + few], self.ne, self.limit)
             return
-        gu = self.gate_up(x, out_dtype=torch.float32)
-        y = torch.empty((n, self.ne * self.inter), dtype=self.rt.dtype, device=dev)
-        ops.moe_act(gu, dense, y, self.limit)
-        self.down(y, out=h, accumulate=accumulate)
+        rank = torch.empty_like(chosen)
+        counts = torch.empty(self.ne, dtype=torch.int32, device=dev)
+        ops.moe_group(chosen, self.ne, rank, counts)
+        per_expert = [int(c) for c in counts.cpu()]          # the step waits for the host here
+        starts = [0]
+        for c in per_expert:
+            starts.append(starts[-1] + c)
+        offsets = torch.tensor(starts[:-1], dtype=torch.int32).to(dev)
+        pairs = n * self.top
+        xs = torch.empty((pairs, self.hidden), dtype=x.dtype, device=dev)
+        ops.moe_gather(x, chosen, rank, offsets, xs)
+        gu = torch.empty((pairs, 2 * self.inter), dtype=torch.float32, device=dev)
+        for e, (gate_up, _) in enumerate(self.experts):
+            if per_expert[e]:
+                gate_up(xs[starts[e]:starts[e + 1]], out=gu[starts[e]:starts[e + 1]])
+        y = torch.empty((pairs, self.inter), dtype=self.rt.dtype, device=dev)
+        ops.moe_act(gu, self._ones(pairs, dev), y, self.limit)
+        rows = torch.empty((pairs, self.hidden), dtype=torch.float32, device=dev)
+        for e, (_, down) in enumerate(self.experts):
+            if per_expert[e]:
+                down(y[starts[e]:starts[e + 1]], out=rows[starts[e]:starts[e + 1]])
+        ops.moe_combine(rows, chosen, rank, offsets, weights, h, accumulate=accumulate)
+
+    def _ones(self, n: int, dev) -> torch.Tensor:
+        """[n][1] ones: the activation kernel's weights where the weighting happens later."""
+        have = getattr(self, "_ones_buf", None)
+        if have is None or have.shape[0] < n:
+            have = self._ones_buf = torch.ones((max(n, 4096), 1), dtype=torch.float32, device=dev)
+        return have[:n]

@@ -490,7 +490,8 @@ def moe_route(x, router, dense, chosen, weights, n_groups, keep):
     top = chosen.shape[1]
     per = E // n_groups
     s = torch.softmax(logits.float(), dim=-1)
-    dense.zero_()
+    if dense is not None:
+        dense.zero_()
     for t in range(n_tok):
         gs = s[t].view(n_groups, per).max(dim=1).values
         kept = torch.argsort(-gs, stable=True)[:keep]
@@ -501,7 +502,8 @@ def moe_route(x, router, dense, chosen, weights, n_groups, keep):
         w = s[t, pick] / (s[t, pick].sum() + 1e-20)
         chosen[t] = pick.to(torch.int32)
         weights[t] = w
-        dense[t, pick] = w
+        if dense is not None:
+            dense[t, pick] = w
 
 
 def _expert_act(g, u, limit):
@@ -520,15 +522,41 @@ def moe_act(gu, dense, out, limit):
 
 def moe_sparse(x, gate_up, down, chosen, weights, out, n_experts, limit):
     n_tok, K = x.shape
-    N, EF = down.shape
-    F = EF // n_experts
+    _, N, F = down.shape
     gu = gate_up.double().view(n_experts, 2, F, K)
-    dn = down.double().view(N, n_experts, F)
+    dn = down.double()
     for t in range(n_tok):
         for k in range(chosen.shape[1]):
             e = int(chosen[t, k])
             y = _expert_act(gu[e, 0] @ x[t].double(), gu[e, 1] @ x[t].double(), limit).to(x.dtype).double()
-            out[t] += (float(weights[t, k]) * (dn[:, e] @ y)).float()
+            out[t] += (float(weights[t, k]) * (dn[e] @ y)).float()
+
+
+def moe_group(chosen, n_experts, rank, counts):
+    seen = [0] * n_experts
+    flat, r = chosen.reshape(-1), rank.view(-1)
+    for p in range(flat.numel()):
+        r[p] = seen[int(flat[p])]
+        seen[int(flat[p])] += 1
+    counts.copy_(torch.tensor(seen, dtype=torch.int32))
+
+
+def _rows_of(chosen, rank, offsets):
+    return (offsets.long()[chosen.long()] + rank.long()).reshape(-1)
+
+
+def moe_gather(x, chosen, rank, offsets, xs):
+    top = chosen.shape[1]
+    xs[_rows_of(chosen, rank, offsets)] = x.repeat_interleave(top, dim=0)
+
+
+def moe_combine(rows, chosen, rank, offsets, weights, out, accumulate=True):
+    n_tok, top = chosen.shape
+    picked = rows[_rows_of(chosen, rank, offsets)].double().view(n_tok, top, -1)
+    acc = out.double() if accumulate else torch.zeros(out.shape, dtype=torch.float64)
+    for k in range(top):
+        acc = acc + weights.double()[:, k, None] * picked[:, k]
+    out.copy_(acc.float())
 
 
 # ------------------------------------------------------------------ sampling
@@ -604,7 +632,7 @@ NAMES = ["embed", "rmsnorm", "gather_rows", "swiglu", "convert", "fill_normal", 
          "group_rmsnorm", "xielu", "rope_table_freqs", "rope_pairs_inplace", "mingru_scan", "latent_prep",
          "headwise_linear", "latent_attn", "headwise_mfma_takes", "headwise_linear_mfma",
          "embed_pos", "gelu_tanh", "weighted_sum", "lightning_scan", "gated_rmsnorm", "rope_half_inplace",
-         "qkv_conv_prep", "capped_attn", "capped_mfma_takes", "capped_attn_prefill", "moe_route", "moe_act", "moe_sparse"]
+         "qkv_conv_prep", "capped_attn", "capped_mfma_takes", "capped_attn_prefill", "moe_route", "moe_act", "moe_sparse", "moe_group", "moe_gather", "moe_combine"]
 
 
 def install(monkeypatch):

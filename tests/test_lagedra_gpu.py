@@ -351,13 +351,30 @@ def test_router_and_experts_kernels():
             plain_ops.moe_act(gu, want[0], y_want, 1.5)
             ops.moe_act(gu.to(DEV), got[0], y, 1.5)
             assert (y.cpu().float() - y_want.float()).abs().max() < tol
-            x, w1, w2 = rnd(n, K, seed=3).to(dtype), (rnd(E * 2 * F, K, seed=4) / 8).to(dtype), (rnd(N, E * F, seed=5) / 5).to(dtype)
+            x, w1, w2 = rnd(n, K, seed=3).to(dtype), (rnd(E, 2 * F, K, seed=4) / 8).to(dtype), (rnd(E, N, F, seed=5) / 5).to(dtype)
             o_want, o = rnd(n, N, seed=6), rnd(n, N, seed=6).to(DEV)
             few = min(n, 16)             # the step sizes the sparse form takes
             plain_ops.moe_sparse(x[:few], w1, w2, want[1][:few], want[2][:few], o_want[:few], E, 1.5)
             ops.moe_sparse(x[:few].contiguous().to(DEV), w1.to(DEV), w2.to(DEV), got[1][:few].contiguous(),
                            got[2][:few].contiguous(), o[:few], E, 1.5)
             assert (o.cpu()[:few] - o_want[:few]).abs().max() < (1e-4 if dtype == torch.float32 else 5e-2)
+        # the grouping of the pairs by expert, the rows side by side and the weighted sums back
+        rank_want, counts_want = torch.empty(n, top, dtype=torch.int32), torch.empty(E, dtype=torch.int32)
+        rank, counts = rank_want.clone().to(DEV), counts_want.clone().to(DEV)
+        plain_ops.moe_group(want[1], E, rank_want, counts_want)
+        ops.moe_group(got[1], E, rank, counts)
+        assert torch.equal(rank.cpu(), rank_want) and torch.equal(counts.cpu(), counts_want) and int(counts_want.sum()) == n * top
+        offsets = torch.cat([torch.zeros(1, dtype=torch.int32), counts_want.cumsum(0)[:-1].to(torch.int32)])
+        xr = rnd(n, 70, seed=8).bfloat16()
+        xs_want, xs = torch.zeros(n * top, 70, dtype=torch.bfloat16), torch.zeros(n * top, 70, dtype=torch.bfloat16, device=DEV)
+        plain_ops.moe_gather(xr, want[1], rank_want, offsets, xs_want)
+        ops.moe_gather(xr.to(DEV), got[1], rank, offsets.to(DEV), xs)
+        assert torch.equal(xs.cpu(), xs_want)
+        rows = rnd(n * top, 50, seed=9)
+        o_want, o = rnd(n, 50, seed=10), rnd(n, 50, seed=10).to(DEV)
+        plain_ops.moe_combine(rows, want[1], rank_want, offsets, want[2], o_want)
+        ops.moe_combine(rows.to(DEV), got[1], rank, offsets.to(DEV), got[2], o)
+        assert (o.cpu() - o_want).abs().max() < 1e-5
 
 
 def test_half_rotation_tables_and_kernel():
