@@ -40,23 +40,16 @@ namespace {
 
 // EPI_XIELU: bfloat16 output of the xIELU activation of (sum + bias); the activation's two constants
 // (a_pos, a_neg: z > 0 -> a_pos z^2 + z/2, else a_neg (e^z - 1 - z) + z/2) stand behind the N biases.
-// EPI_GELU: bfloat16 output of gelu (tanh form) of (sum + bias).
-enum { EPI_F32 = 0, EPI_ACC_F32 = 1, EPI_BF16 = 2, EPI_SWIGLU = 3, EPI_XIELU = 4, EPI_GELU = 5 };
+enum { EPI_F32 = 0, EPI_ACC_F32 = 1, EPI_BF16 = 2, EPI_SWIGLU = 3, EPI_XIELU = 4 };
 
 __device__ __forceinline__ float xielu_f(float z, float a_pos, float a_neg) {
   return z > 0.f ? fmaf(a_pos * z, z, 0.5f * z) : fmaf(a_neg, expm1f(z) - z, 0.5f * z);
-}
-
-__device__ __forceinline__ float gelu_tanh_f(float z) {
-  return 0.5f * z * (1.0f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
 }
 
 __device__ __forceinline__ void store_out(void* C, int ldc, int m, int n, float v, int epi,
                                           const float* __restrict__ bias = nullptr, int N = 0) {
   if (epi == EPI_XIELU) {
     ((bf16*)C)[(size_t)m * ldc + n] = (bf16)xielu_f(v, bias[N], bias[N + 1]);
-  } else if (epi == EPI_GELU) {
-    ((bf16*)C)[(size_t)m * ldc + n] = (bf16)gelu_tanh_f(v);
   } else if (epi == EPI_BF16) {
     ((bf16*)C)[(size_t)m * ldc + n] = (bf16)v;
   } else {
@@ -1691,8 +1684,6 @@ __global__ __launch_bounds__(256) void skinny_reduce_kernel(const float* __restr
     v = sum_of_parts(part, stride, (size_t)m * N + n, splits) * rf + (bias ? bias[n] : 0.f);
     if (epi == EPI_XIELU) {
       ((bf16*)C)[(size_t)m * ldc + n] = (bf16)xielu_f(v, bias[N], bias[N + 1]);
-    } else if (epi == EPI_GELU) {
-      ((bf16*)C)[(size_t)m * ldc + n] = (bf16)gelu_tanh_f(v);
     } else if (epi == EPI_BF16) {
       ((bf16*)C)[(size_t)m * ldc + n] = (bf16)v;
     } else {
@@ -1756,10 +1747,6 @@ __global__ __launch_bounds__(256) void skinny_reduce4_kernel(const float* __rest
       bf16* c = (bf16*)C + (size_t)m * ldc + n;
       c[0] = (bf16)xielu_f(v.x, ap, an); c[1] = (bf16)xielu_f(v.y, ap, an);
       c[2] = (bf16)xielu_f(v.z, ap, an); c[3] = (bf16)xielu_f(v.w, ap, an);
-    } else if (epi == EPI_GELU) {
-      bf16* c = (bf16*)C + (size_t)m * ldc + n;
-      c[0] = (bf16)gelu_tanh_f(v.x); c[1] = (bf16)gelu_tanh_f(v.y);
-      c[2] = (bf16)gelu_tanh_f(v.z); c[3] = (bf16)gelu_tanh_f(v.w);
     } else if (epi == EPI_BF16) {
       bf16* c = (bf16*)C + (size_t)m * ldc + n;
       c[0] = (bf16)v.x; c[1] = (bf16)v.y; c[2] = (bf16)v.z; c[3] = (bf16)v.w;
@@ -1917,7 +1904,7 @@ TilePlan plan_tiles(int M, int N, int K, bool dma_ok, int epi, int n_cu) {
   const long cu = n_cu > 0 ? n_cu : 1;
   const long nkt = (K + 63) / 64, chunks = (K + 255) / 256;
   const double mn = (double)M * (double)N;
-  const double epi_us = (epi == EPI_ACC_F32 ? 8. : epi == EPI_F32 ? 4. : (epi == EPI_BF16 || epi == EPI_XIELU || epi == EPI_GELU) ? 2. : 1.) * mn / 4e6;
+  const double epi_us = (epi == EPI_ACC_F32 ? 8. : epi == EPI_F32 ? 4. : (epi == EPI_BF16 || epi == EPI_XIELU) ? 2. : 1.) * mn / 4e6;
   const double start_us = 12.;
   auto tiles = [&](int bm, int bn) { return (long)((M + bm - 1) / bm) * ((N + bn - 1) / bn); };
   auto cut = [&](long parts, int& splits, int& per) {          // K in `parts` runs of whole chunks of 256
@@ -1995,7 +1982,7 @@ SkinnyChoice skinny_choice(int M, int N, int K, bool aligned, int epi, int split
 MF_API int mf_gemm_bf16(const void* A, int lda, const void* W, int ldw, const float* bias, void* C,
                         int ldc, int M, int N, int K, int epi, int variant, hipStream_t stream) {
   if (M <= 0 || N <= 0) return 0;
-  if (K <= 0 || lda < K || ldw < K || epi < 0 || epi > EPI_GELU || (epi == EPI_XIELU && !bias)) return (int)hipErrorInvalidValue;
+  if (K <= 0 || lda < K || ldw < K || epi < 0 || epi > EPI_XIELU || (epi == EPI_XIELU && !bias)) return (int)hipErrorInvalidValue;
   if (epi == EPI_SWIGLU ? (N % 64 != 0 || ldc > N / 2 || ldc <= N / 2 - 32 || bias) : ldc < N)
     return (int)hipErrorInvalidValue;
   const int vec_ok = (lda % 8 == 0) && (ldw % 8 == 0) && ((uintptr_t)A % 16 == 0) &&
@@ -2037,7 +2024,7 @@ MF_API int mf_gemm_bf16_splitk(const void* A, int lda, const void* W, int ldw, c
                                int ldc, float* part, int M, int N, int K, int splits, int k_per_split,
                                int epi, int variant, hipStream_t stream) {
   if (M <= 0 || N <= 0) return 0;
-  if (K <= 0 || lda < K || ldw < K || epi < 0 || epi > EPI_GELU || (epi == EPI_XIELU && !bias) || splits < 2 || !part || k_per_split % 64 != 0 ||
+  if (K <= 0 || lda < K || ldw < K || epi < 0 || epi > EPI_XIELU || (epi == EPI_XIELU && !bias) || splits < 2 || !part || k_per_split % 64 != 0 ||
       (long)splits * k_per_split < K || (long)(splits - 1) * k_per_split >= K)
     return (int)hipErrorInvalidValue;
   if (epi == EPI_SWIGLU ? (N % 64 != 0 || ldc > N / 2 || ldc <= N / 2 - 32 || bias) : ldc < N)
@@ -2093,7 +2080,7 @@ static int skinny_product(const void* A, int lda, const void* W, const void* Wt,
                           void* C, int ldc, float* part, int M, int N, int K, int splits, int k_per_split, int epi,
                           const FusedNorm& fused, hipStream_t stream) {
   if (M <= 0 || N <= 0) return 0;
-  if (M > 64 || K <= 0 || lda < K || ldw < K || epi < 0 || epi > EPI_GELU || (epi == EPI_XIELU && !bias) || splits < 1 ||
+  if (M > 64 || K <= 0 || lda < K || ldw < K || epi < 0 || epi > EPI_XIELU || (epi == EPI_XIELU && !bias) || splits < 1 ||
       k_per_split % KC != 0 || (long)splits * k_per_split < K || (splits > 1 && !part))
     return (int)hipErrorInvalidValue;
   if (epi == EPI_SWIGLU ? (N % 64 != 0 || ldc > N / 2 || ldc <= N / 2 - 32 || bias || (M > 16 && !part))
@@ -2172,7 +2159,7 @@ MF_API int mf_gemm_bf16_normed(const float* x, int ldx, const int* row_idx, cons
                                const void* W, const void* Wt, int ldw, const float* bias, void* C, int ldc, int M,
                                int N, int K, int epi, hipStream_t stream) {
   if (M <= 0 || N <= 0) return 0;
-  if (K <= 0 || epi < 0 || epi > EPI_GELU || (epi == EPI_XIELU && !bias)) return (int)hipErrorInvalidValue;
+  if (K <= 0 || epi < 0 || epi > EPI_XIELU || (epi == EPI_XIELU && !bias)) return (int)hipErrorInvalidValue;
   if (ldx % 4 != 0 || ldw % 8 != 0 || (uintptr_t)x % 16 != 0 || (uintptr_t)g % 16 != 0 || (uintptr_t)W % 16 != 0)
     return MF_NOT_BUILT;
   const NormArgs norm{g, row_idx, eps};
@@ -2184,7 +2171,7 @@ MF_API int mf_gemm_bf16_normed(const float* x, int ldx, const int* row_idx, cons
 // for mf_gemm_bf16_splitk with out[1] splits of out[2] of K each.  `aligned`: 16-byte aligned
 // operands with row strides and K in multiples of 8.
 MF_API int mf_gemm_bf16_tile_plan(int M, int N, int K, int aligned, int epi, int n_cu, int* out) {
-  if (!out || M <= 0 || N <= 0 || K <= 0 || epi < 0 || epi > EPI_GELU || n_cu <= 0) return (int)hipErrorInvalidValue;
+  if (!out || M <= 0 || N <= 0 || K <= 0 || epi < 0 || epi > EPI_XIELU || n_cu <= 0) return (int)hipErrorInvalidValue;
   const bool dma_ok = aligned && K % DMA_BK == 0 && (size_t)M * K * 2 < (1ull << 32) && (size_t)N * K * 2 < (1ull << 32);
   const TilePlan plan = plan_tiles(M, N, K, dma_ok, epi, n_cu);
   out[0] = plan.variant;
@@ -2200,7 +2187,7 @@ MF_API int mf_gemm_bf16_tile_plan(int M, int N, int K, int aligned, int epi, int
 // such kernel": norm and product run one after the other); `n_cu`: compute units of the device.
 MF_API int mf_gemm_bf16_plan(int M, int N, int K, int aligned, int epi, int splits, int k_per_split,
                              int normed, int n_cu, char* name, int cap) {
-  if (!name || cap < 48 || M <= 0 || N <= 0 || K <= 0 || epi < 0 || epi > EPI_GELU || n_cu <= 0) return (int)hipErrorInvalidValue;
+  if (!name || cap < 48 || M <= 0 || N <= 0 || K <= 0 || epi < 0 || epi > EPI_XIELU || n_cu <= 0) return (int)hipErrorInvalidValue;
   const char* what = "";
   if (normed) {
     what = (aligned && stationary_takes(M, N, K, epi, true)) ? "stationary16_kernel(norm)" : "";

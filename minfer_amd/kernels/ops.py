@@ -19,7 +19,7 @@ PAGE = 64          # tokens per cache page (MF_PAGE in csrc/common.h)
 HAVE_PREFILL_ATTENTION = True
 PREFILL_MAX_SHARES = 8  # workgroups that may take the pages of one block of queries of the prompt attention in turn
 PREFILL_MIN_PAGES = 4   # ... each with at least this many pages
-EPI_F32, EPI_ACC_F32, EPI_BF16, EPI_SWIGLU, EPI_XIELU, EPI_GELU = 0, 1, 2, 3, 4, 5
+EPI_F32, EPI_ACC_F32, EPI_BF16, EPI_SWIGLU, EPI_XIELU = 0, 1, 2, 3, 4
 
 
 class KernelError(RuntimeError):
@@ -1181,11 +1181,10 @@ def _need_tiled(tiled: Optional[torch.Tensor], name: str, n: int, k: int) -> Non
 
 def linear(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor], out: torch.Tensor,
            accumulate: bool = False, variant: int = 0, tiled: Optional[torch.Tensor] = None,
-           xielu: bool = False, gelu: bool = False) -> None:
+           xielu: bool = False) -> None:
     """out (+)= x @ weight^T (+ bias).  weight is [out][in].  float32 weights take the true
     32-bit kernel; bfloat16 weights take the matrix-core kernels (a few rows: the streaming
-    kernel).  `out` is float32, or bfloat16 for a bfloat16 product that is stored; `gelu`: the stored
-    values are gelu (tanh form) of the sums.  `tiled`:
+    kernel).  `out` is float32, or bfloat16 for a bfloat16 product that is stored.  `tiled`:
     `tile_weight(weight)`, which the kernels for at most 64 rows read instead where they can."""
     _need(x, "linear.x", _FLOATS)
     _need(weight, "linear.weight", x.dtype)
@@ -1200,8 +1199,6 @@ def linear(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor], 
         _need(bias, "linear.bias", torch.float32, (n + 2,))
     elif bias is not None:
         _need(bias, "linear.bias", torch.float32, (n,))
-    if gelu and (x.dtype != torch.bfloat16 or out.dtype != torch.bfloat16 or accumulate or xielu):
-        raise KernelError("linear(gelu): needs bfloat16 operands and output")
     if m == 0:
         return
     if x.dtype == torch.float32:
@@ -1211,7 +1208,7 @@ def linear(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor], 
         return
     if accumulate and out.dtype != torch.float32:
         raise KernelError("linear: accumulation needs a float32 output")
-    epi = EPI_XIELU if xielu else EPI_GELU if gelu else (EPI_BF16 if out.dtype == torch.bfloat16 else (EPI_ACC_F32 if accumulate else EPI_F32))
+    epi = EPI_XIELU if xielu else (EPI_BF16 if out.dtype == torch.bfloat16 else (EPI_ACC_F32 if accumulate else EPI_F32))
     aligned = not (x.data_ptr() % 16 or weight.data_ptr() % 16 or k % 8)
     if m <= 64 and variant == 0:
         splits, per = _k_split(m, n, k, False, aligned, tiled=tiled is not None)

@@ -126,7 +126,7 @@ class DenseXIELU(FeedForward):
 @register_feed_forward("dense_gelu")
 class DenseGelu(FeedForward):
     """down(gelu(up x)) without biases, gelu in its tanh form, from the up product's 32-bit sums and
-    rounded once (in bfloat16 inside the product's epilogue).  params: hidden_size, intermediate_size, up, down (tensor names)."""
+    rounded once.  params: hidden_size, intermediate_size, up, down (tensor names)."""
 
     takes_normed = True
     can_overwrite = True
@@ -149,12 +149,7 @@ class DenseGelu(FeedForward):
         return self.up.decode_copy(make, min_row_length) + self.down.decode_copy(make, min_row_length)
 
     def forward(self, x, h, ctx, accumulate: bool = True) -> None:
-        if isinstance(x, Normed):
-            x = x.tensor()
-        y = torch.empty((x.shape[0], self.inter), dtype=self.rt.dtype, device=x.device)
-        if x.dtype == torch.bfloat16 and self.up.weight.dtype == torch.bfloat16:
-            # the activation from the product's 32-bit sums, in its epilogue
-            ops.linear(x, self.up.weight, None, y, tiled=self.up.tiled, gelu=True)
-        else:
-            ops.gelu_tanh(self.up(x, out_dtype=torch.float32), y)
+        u = self.up(x, out_dtype=torch.float32)
+        y = torch.empty((u.shape[0], self.inter), dtype=self.rt.dtype, device=u.device)
+        ops.gelu_tanh(u, y)
         self.down(y, out=h, accumulate=accumulate)

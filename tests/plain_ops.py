@@ -99,12 +99,8 @@ def rope_inplace(qkv, cos, sin, positions, n_rot_heads, n_heads_total, head_dim)
     x[:, :n_rot_heads] = torch.cat([v0 * c - v1 * s, v0 * s + v1 * c], dim=-1).float()
 
 
-def linear(x, weight, bias, out, accumulate=False, variant=0, tiled=None, xielu=False, gelu=False):
+def linear(x, weight, bias, out, accumulate=False, variant=0, tiled=None, xielu=False):
     y = x.double() @ weight.double().t()
-    if gelu:
-        y = y if bias is None else y + bias.double()
-        out.copy_((0.5 * y * (1.0 + torch.tanh(math.sqrt(2.0 / math.pi) * (y + 0.044715 * y ** 3)))).to(out.dtype))
-        return
     if xielu:                            # the activation's constants ride behind the biases
         n = weight.shape[0]
         y = y + bias[:n].double()

@@ -131,17 +131,6 @@ def test_position_rows_gelu_and_weighted_sums():
         assert (got.cpu() - want).abs().max() < 1e-5
 
 
-@pytest.mark.parametrize("m, n, k", [(1, 112, 96), (8, 8192, 2048), (40, 200, 128), (300, 384, 256), (2048, 1000, 136)])
-def test_product_with_gelu_epilogue(m, n, k):
-    """Every size class of the bfloat16 product (few rows, 17 to 64, tiles) stores gelu of its 32-bit sums."""
-    from minfer_amd.kernels import ops
-    x, w = rnd(m, k, seed=1).bfloat16(), (rnd(n, k, seed=2) / k ** 0.5).bfloat16()
-    want, got = torch.empty(m, n, dtype=torch.bfloat16), torch.empty(m, n, dtype=torch.bfloat16, device=DEV)
-    plain_ops.linear(x, w, None, want, gelu=True)
-    ops.linear(x.to(DEV), w.to(DEV), None, got, gelu=True)
-    assert (got.cpu().float() - want.float()).abs().max() < 3e-2
-
-
 @pytest.mark.parametrize("heads, dim, vdim, lens", [(3, 20, 12, (1, 5, 200, 64, 129)), (1, 40, 72, (700,)),
                                                     (2, 136, 16, (3, 128, 65)), (3, 5, 7, (1, 1, 1)), (2, 128, 130, (300, 2))])
 def test_lightning_scan_kernels(heads, dim, vdim, lens):
