@@ -14,9 +14,10 @@
 // into LDS, then rotation, blending, the cache write and q rounded to the run type.
 // `conv_state_update_kernel`: behind it, the sequences' new last rows.
 // `capped_attn_kernel`: a workgroup owns (token, kv head, up to 8 query heads of its group, key
-// split) and walks the token's keys 256 at a time: a thread forms the scores of one key for all the
-// heads (phase 1), a wave takes the maximum, the exponentials and their sum of a head (phase 2), and
-// the threads, as (key residue, value column) pairs, add the weighted value rows (phase 3).  Every
+// split) and walks the token's keys 256 at a time, from the half page of its first key on: a thread forms
+// the scores of one key for all the heads (phase 1), a wave takes the maximum, the exponentials and their
+// sum of a head (phase 2), and the threads, as (key residue, value column) pairs, add the weighted value
+// rows (phase 3; in bfloat16 a thread takes a column's 32 keys of a half page with four 16-byte loads).  Every
 // size is a run-time number; all sums are 32-bit and their order is fixed.
 #include "attn_tokens_impl.h"
 
@@ -158,50 +159,58 @@ __global__ __launch_bounds__(256) void capped_attn_kernel(
   const float inv_cap = cap > 0.f ? 1.0f / cap : 0.f;
   __syncthreads();
 
-  for (int c0 = j_begin; c0 < j_end; c0 += MF_CAP_KEYS) {
-    const int nkeys = min(MF_CAP_KEYS, j_end - c0);
-    // phase 1: the scores of key c0 + thread
-    if (threadIdx.x < nkeys) {
-      const int j = c0 + threadIdx.x;
-      const T* krow = kc + (((size_t)pt[j / MF_PAGE] * nk + hk) * MF_PAGE + j % MF_PAGE) * D;
+  // rounds of 256 keys from the half page of the first key on: a round's 32-key groups are half pages
+  for (int cb = j_begin < j_end ? (j_begin & ~31) : j_end; cb < j_end; cb += MF_CAP_KEYS) {       // (a split may be empty)
+    // phase 1: the scores of key cb + thread (-inf outside the token's keys)
+    {
+      const int j = cb + threadIdx.x;
+      const bool valid = j >= j_begin && j < j_end;
       float s[MF_CAP_GC];
 #pragma unroll
       for (int g = 0; g < MF_CAP_GC; ++g) s[g] = 0.f;
-      if ((D * sizeof(T)) % 16 == 0) {
-        constexpr int PER = 16 / sizeof(T);
-        for (int d = 0; d < D; d += PER) {
-          alignas(16) T kv[PER];
-          *(uint4*)kv = *(const uint4*)(krow + d);
+      if (valid) {
+        const T* krow = kc + (((size_t)pt[j / MF_PAGE] * nk + hk) * MF_PAGE + j % MF_PAGE) * D;
+        if ((D * sizeof(T)) % 16 == 0) {
+          constexpr int PER = 16 / sizeof(T);
+          for (int d0 = 0; d0 < D; d0 += 4 * PER) {        // four loads in flight
+            alignas(16) T kv[4][PER];
 #pragma unroll
-          for (int e = 0; e < PER; ++e) {
-            const float kf = to_f32(kv[e]);
+            for (int c = 0; c < 4; ++c)
+              if (d0 + c * PER < D) *(uint4*)kv[c] = *(const uint4*)(krow + d0 + c * PER);
 #pragma unroll
-            for (int g = 0; g < MF_CAP_GC; ++g) s[g] = fmaf(sq[g * D + d + e], kf, s[g]);
+            for (int c = 0; c < 4; ++c) {
+              if (d0 + c * PER >= D) break;
+#pragma unroll
+              for (int e = 0; e < PER; ++e) {
+                const float kf = to_f32(kv[c][e]);
+#pragma unroll
+                for (int g = 0; g < MF_CAP_GC; ++g) s[g] = fmaf(sq[g * D + d0 + c * PER + e], kf, s[g]);
+              }
+            }
           }
-        }
-      } else {
-        for (int d = 0; d < D; ++d) {
-          const float kf = to_f32(krow[d]);
+        } else {
+          for (int d = 0; d < D; ++d) {
+            const float kf = to_f32(krow[d]);
 #pragma unroll
-          for (int g = 0; g < MF_CAP_GC; ++g) s[g] = fmaf(sq[g * D + d], kf, s[g]);
+            for (int g = 0; g < MF_CAP_GC; ++g) s[g] = fmaf(sq[g * D + d], kf, s[g]);
+          }
         }
       }
 #pragma unroll
       for (int g = 0; g < MF_CAP_GC; ++g) {
         float x = s[g] * tm[g];
         if (cap > 0.f) x = cap * tanhf(x * inv_cap);
-        sc[g * MF_CAP_KEYS + threadIdx.x] = x;
+        sc[g * MF_CAP_KEYS + threadIdx.x] = valid ? x : -INFINITY;
       }
     }
     __syncthreads();
-    // phase 2: wave w takes the heads w, w + 4
+    // phase 2: wave w takes the heads w, w + 4; every round holds at least one of the token's keys
     for (int g = w; g < gcount; g += 4) {
       float x[MF_CAP_KEYS / 64];
       float mx = -INFINITY;
 #pragma unroll
       for (int r = 0; r < MF_CAP_KEYS / 64; ++r) {
-        const int i = lane + 64 * r;
-        x[r] = i < nkeys ? sc[g * MF_CAP_KEYS + i] : -INFINITY;
+        x[r] = sc[g * MF_CAP_KEYS + lane + 64 * r];
         mx = fmaxf(mx, x[r]);
       }
       mx = wave_max(mx);
@@ -210,9 +219,8 @@ __global__ __launch_bounds__(256) void capped_attn_kernel(
       float sum = 0.f;
 #pragma unroll
       for (int r = 0; r < MF_CAP_KEYS / 64; ++r) {
-        const int i = lane + 64 * r;
-        const float pe = i < nkeys ? attn_tokens::exp_for<T>(x[r] - m_new) : 0.f;
-        if (i < nkeys) sc[g * MF_CAP_KEYS + i] = pe;
+        const float pe = x[r] == -INFINITY ? 0.f : attn_tokens::exp_for<T>(x[r] - m_new);
+        sc[g * MF_CAP_KEYS + lane + 64 * r] = pe;
         sum += pe;
       }
       sum = wave_sum(sum);
@@ -224,15 +232,35 @@ __global__ __launch_bounds__(256) void capped_attn_kernel(
       }
     }
     __syncthreads();
-    // phase 3: thread (ks, v) adds the value rows of the keys ks, ks + KS, ...
+    // phase 3: thread (ks, v) adds the value rows.  bfloat16 pages keep a value column's 32 keys of a half
+    // page side by side: a thread takes whole half pages, 16 bytes a load; 32-bit pages are read key by key.
     if (v < V) {
 #pragma unroll
       for (int g = 0; g < MF_CAP_GC; ++g) acc[g] *= sm_corr[g];
-      for (int i = ks; i < nkeys; i += KS) {
-        const int j = c0 + i;
-        const float vv = v_elem<T>(vc, pt[j / MF_PAGE], nk, hk, j % MF_PAGE, V, v);
+      if (sizeof(T) == 2) {
+        for (int gi = ks; gi < MF_CAP_KEYS / 32; gi += KS) {
+          const int jb = cb + 32 * gi;
+          if (jb >= j_end || jb + 32 <= j_begin) continue;
+          const T* vrow = vc + ((((size_t)pt[jb / MF_PAGE] * nk + hk) * 2 + (jb / 32 & 1)) * V + v) * 32;
+          alignas(16) T vals[32];
 #pragma unroll
-        for (int g = 0; g < MF_CAP_GC; ++g) acc[g] = fmaf(sc[g * MF_CAP_KEYS + i], vv, acc[g]);
+          for (int c = 0; c < 4; ++c) *(uint4*)(vals + 8 * c) = *(const uint4*)(vrow + 8 * c);
+#pragma unroll
+          for (int i = 0; i < 32; ++i) {
+            const int j = jb + i;
+            const float vv = (j >= j_begin && j < j_end) ? to_f32(vals[i]) : 0.f;      // unwritten keys may hold anything
+#pragma unroll
+            for (int g = 0; g < MF_CAP_GC; ++g) acc[g] = fmaf(sc[g * MF_CAP_KEYS + 32 * gi + i], vv, acc[g]);
+          }
+        }
+      } else {
+        for (int i = ks; i < MF_CAP_KEYS; i += KS) {
+          const int j = cb + i;
+          if (j < j_begin || j >= j_end) continue;
+          const float vv = v_elem<T>(vc, pt[j / MF_PAGE], nk, hk, j % MF_PAGE, V, v);
+#pragma unroll
+          for (int g = 0; g < MF_CAP_GC; ++g) acc[g] = fmaf(sc[g * MF_CAP_KEYS + i], vv, acc[g]);
+        }
       }
     }
     __syncthreads();
