@@ -228,64 +228,48 @@ __global__ __launch_bounds__(256) void moe_sparse_up_kernel(const WT* __restrict
   }
 }
 
-// down [E][N][F], y [tokens][top][F]:
-// out[t][n] += sum_k w[t][k] dot(down[e_k][n], y[t][k]), a token's choices added in their order.
-// A wave owns output n: for every expert that has pairs, its part of row n is read once and meets the y rows
-// of the expert's pairs; lane p % 64 keeps pair p's dot product until the tokens' sums are formed.
+// down [E][N][F], y [tokens][top][F] -> rows[pair][N]: the pairs' outputs, not yet weighted.  A wave owns
+// (expert, n): the expert's row n is read once and meets the y rows of the expert's pairs.  The tokens' sums
+// are formed behind it (`moe_combine_kernel`, a token's choices in their order).
 template <typename WT>
 __global__ __launch_bounds__(256) void moe_sparse_down_kernel(const WT* __restrict__ y, const WT* __restrict__ down,
-                                                              const int* __restrict__ chosen,
-                                                              const float* __restrict__ weights, float* __restrict__ out,
-                                                              int n_tok, int top, int E, int F, int N) {
+                                                              const int* __restrict__ chosen, float* __restrict__ rows,
+                                                              int n_pairs, int F, int N) {
+  const int e = blockIdx.x;
   const int lane = threadIdx.x & 63;
-  const int n = blockIdx.x * 4 + (threadIdx.x >> 6);
-  if (n >= N) return;
-  const int n_pairs = n_tok * top;
+  const int n = blockIdx.y * 4 + (threadIdx.x >> 6);
   const int c0 = lane < n_pairs ? chosen[lane] : -1, c1 = lane + 64 < n_pairs ? chosen[lane + 64] : -1;
+  const unsigned long long mine0 = __ballot(c0 == e), mine1 = __ballot(c1 == e);
+  if (!(mine0 | mine1) || n >= N) return;
+  const WT* wr = down + ((size_t)e * N + n) * F;
   const bool vec = (F * sizeof(WT)) % 16 == 0;
-  float dot0 = 0.f, dot1 = 0.f;          // of pair lane, of pair lane + 64
-  for (int i = 0; i < n_pairs; ++i) {
-    const int e = chosen[i];
-    const unsigned long long mine0 = __ballot(c0 == e), mine1 = __ballot(c1 == e);
-    const unsigned long long before0 = i < 64 ? (i ? ~0ull >> (64 - i) : 0ull) : ~0ull;
-    const unsigned long long before1 = i <= 64 ? 0ull : ~0ull >> (128 - i);
-    if ((mine0 & before0) | (mine1 & before1)) continue;       // an earlier pair led this expert
-    const WT* wr = down + ((size_t)e * N + n) * F;
-    float acc[MF_MOE_SPARSE_TOKENS];
+  float acc[MF_MOE_SPARSE_TOKENS];
 #pragma unroll
-    for (int j = 0; j < MF_MOE_SPARSE_TOKENS; ++j) acc[j] = 0.f;
-    for (int k = lane * 8; k < F; k += 512) {
-      float wv[8];
-      load8(wr + k, vec, F - k, wv);
-      unsigned long long m0 = mine0, m1 = mine1;
-#pragma unroll
-      for (int j = 0; j < MF_MOE_SPARSE_TOKENS; ++j) {
-        if (m0 | m1) {
-          const int pr = next_pair(m0, m1);
-          float yv[8];
-          load8(y + (size_t)pr * F + k, vec, F - k, yv);
-#pragma unroll
-          for (int q = 0; q < 8; ++q) acc[j] = fmaf(wv[q], yv[q], acc[j]);
-        }
-      }
-    }
+  for (int j = 0; j < MF_MOE_SPARSE_TOKENS; ++j) acc[j] = 0.f;
+  for (int k = lane * 8; k < F; k += 512) {
+    float wv[8];
+    load8(wr + k, vec, F - k, wv);
     unsigned long long m0 = mine0, m1 = mine1;
 #pragma unroll
     for (int j = 0; j < MF_MOE_SPARSE_TOKENS; ++j) {
       if (m0 | m1) {
         const int pr = next_pair(m0, m1);
-        const float v = wave_sum(acc[j]);
-        if (lane == (pr & 63)) { if (pr < 64) dot0 = v; else dot1 = v; }
+        float yv[8];
+        load8(y + (size_t)pr * F + k, vec, F - k, yv);
+#pragma unroll
+        for (int q = 0; q < 8; ++q) acc[j] = fmaf(wv[q], yv[q], acc[j]);
       }
     }
   }
-  float total = 0.f;
-  for (int k = 0; k < top; ++k) {
-    const int pr = min(lane, n_tok - 1) * top + k;       // lanes behind the tokens repeat the last one's work
-    const float d0 = __shfl(dot0, pr & 63, MF_WAVE), d1 = __shfl(dot1, pr & 63, MF_WAVE);
-    total = fmaf(weights[pr], pr < 64 ? d0 : d1, total);
+  unsigned long long m0 = mine0, m1 = mine1;
+#pragma unroll
+  for (int j = 0; j < MF_MOE_SPARSE_TOKENS; ++j) {
+    if (m0 | m1) {
+      const int pr = next_pair(m0, m1);
+      const float v = wave_sum(acc[j]);
+      if (lane == 0) rows[(size_t)pr * N + n] = v;
+    }
   }
-  if (lane < n_tok) out[(size_t)lane * N + n] += total;
 }
 
 // ------------------------------------------------------------------ many tokens: the tokens of an expert together
@@ -336,7 +320,8 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(const float* __restric
   float a = add ? out[(size_t)t * N + i] : 0.f;
   for (int k = 0; k < top; ++k) {
     const int p = t * top + k;
-    a = fmaf(weights[p], rows[(size_t)(offsets[chosen[p]] + rank[p]) * N + i], a);
+    const int row = offsets ? offsets[chosen[p]] + rank[p] : p;      // without offsets: pair p's row is row p
+    a = fmaf(weights[p], rows[(size_t)row * N + i], a);
   }
   out[(size_t)t * N + i] = a;
 }
@@ -369,23 +354,28 @@ MF_API int mf_moe_act(const float* gu, const float* dense, void* y, int y_is_bf1
 }
 
 MF_API int mf_moe_sparse(const void* x, const void* gate_up, const void* down, const int* chosen, const float* weights,
-                         void* y, float* out, int is_bf16, int n_tok, int top, int E, int F, int K, int N, float limit,
-                         hipStream_t stream) {
+                         void* y, float* rows, float* out, int is_bf16, int n_tok, int top, int E, int F, int K, int N,
+                         float limit, hipStream_t stream) {
   if (n_tok <= 0) return 0;
-  if (top <= 0 || E <= 0 || F <= 0 || K <= 0 || N <= 0 || n_tok > MF_MOE_SPARSE_TOKENS || n_tok * top > MF_MOE_SPARSE_PAIRS)
+  if (top <= 0 || E <= 0 || F <= 0 || K <= 0 || N <= 0 || n_tok > MF_MOE_SPARSE_TOKENS || n_tok * top > MF_MOE_SPARSE_PAIRS ||
+      !y || !rows)
     return (int)hipErrorInvalidValue;
-  dim3 g1(E, (F + 3) / 4), g2((N + 3) / 4);
+  dim3 g1(E, (F + 3) / 4), g2(E, (N + 3) / 4);
+  const int pairs = n_tok * top;
   if (is_bf16) {
-    moe_sparse_up_kernel<bf16><<<g1, 256, 0, stream>>>((const bf16*)x, (const bf16*)gate_up, chosen, (bf16*)y, n_tok * top, top, F, K, limit);
+    moe_sparse_up_kernel<bf16><<<g1, 256, 0, stream>>>((const bf16*)x, (const bf16*)gate_up, chosen, (bf16*)y, pairs, top, F, K, limit);
     int rc = mf_launch_status();
     if (rc) return rc;
-    moe_sparse_down_kernel<bf16><<<g2, 256, 0, stream>>>((const bf16*)y, (const bf16*)down, chosen, weights, out, n_tok, top, E, F, N);
+    moe_sparse_down_kernel<bf16><<<g2, 256, 0, stream>>>((const bf16*)y, (const bf16*)down, chosen, rows, pairs, F, N);
   } else {
-    moe_sparse_up_kernel<float><<<g1, 256, 0, stream>>>((const float*)x, (const float*)gate_up, chosen, (float*)y, n_tok * top, top, F, K, limit);
+    moe_sparse_up_kernel<float><<<g1, 256, 0, stream>>>((const float*)x, (const float*)gate_up, chosen, (float*)y, pairs, top, F, K, limit);
     int rc = mf_launch_status();
     if (rc) return rc;
-    moe_sparse_down_kernel<float><<<g2, 256, 0, stream>>>((const float*)y, (const float*)down, chosen, weights, out, n_tok, top, E, F, N);
+    moe_sparse_down_kernel<float><<<g2, 256, 0, stream>>>((const float*)y, (const float*)down, chosen, rows, pairs, F, N);
   }
+  int rc = mf_launch_status();
+  if (rc) return rc;
+  moe_combine_kernel<<<dim3(n_tok, (N + 255) / 256), 256, 0, stream>>>(rows, chosen, nullptr, nullptr, weights, out, top, N, 1);
   return mf_launch_status();
 }
 

@@ -67,7 +67,7 @@ _PROTOTYPES = {
     "moe": {
         "mf_moe_route": [_P, c_int, _P, c_int, _P, _P, _P, c_int, c_int, c_int, c_int, c_int, _P],
         "mf_moe_act": [_P, _P, _P, c_int, c_int, c_int, c_int, c_float, _P],
-        "mf_moe_sparse": [_P, _P, _P, _P, _P, _P, _P, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, _P],
+        "mf_moe_sparse": [_P, _P, _P, _P, _P, _P, _P, _P, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, _P],
         "mf_moe_group": [_P, c_int, c_int, _P, _P, _P],
         "mf_moe_gather": [_P, c_int, _P, _P, _P, _P, c_int, c_int, c_int, _P],
         "mf_moe_combine": [_P, _P, _P, _P, _P, _P, c_int, c_int, c_int, c_int, _P],
@@ -849,7 +849,8 @@ def moe_sparse(x: torch.Tensor, gate_up: torch.Tensor, down: torch.Tensor, chose
         raise KernelError(f"moe_sparse: {n_tok} tokens with {top} experts each; it takes {MOE_SPARSE_TOKENS} tokens and "
                           f"{MOE_SPARSE_PAIRS} pairs")
     y = torch.empty((n_tok, top, F), dtype=x.dtype, device=x.device)
-    _check(_fn("moe", "mf_moe_sparse")(_ptr(x), _ptr(gate_up), _ptr(down), _ptr(chosen), _ptr(weights), _ptr(y), _ptr(out),
+    rows = torch.empty((n_tok * top, N), dtype=torch.float32, device=x.device)
+    _check(_fn("moe", "mf_moe_sparse")(_ptr(x), _ptr(gate_up), _ptr(down), _ptr(chosen), _ptr(weights), _ptr(y), _ptr(rows), _ptr(out),
                                         _is_bf16(x), n_tok, top, n_experts, F, K, N, float(limit), _stream()), "moe_sparse")
 
 SCAN_CHUNK = 32          # tokens of a chunk of the chunked scan (MF_SCAN_CHUNK in csrc/recurrence.hip)
