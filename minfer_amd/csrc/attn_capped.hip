@@ -117,31 +117,6 @@ __device__ __forceinline__ float v_elem(const T* __restrict__ vc, int page, int 
   return to_f32(vc[(((size_t)page * nk + hk) * MF_PAGE + in_page) * V + e]);
 }
 
-// the scores of one key row against the first NG of the staged query heads
-template <typename T, int NG>
-__device__ __forceinline__ void key_scores(const T* __restrict__ krow, const float* __restrict__ sq, int D,
-                                           float (&s)[MF_CAP_GC]) {
-  if ((D * sizeof(T)) % 16 == 0) {
-    constexpr int PER = 16 / sizeof(T);
-    for (int d = 0; d < D; d += PER) {
-      alignas(16) T kv[PER];
-      *(uint4*)kv = *(const uint4*)(krow + d);
-#pragma unroll
-      for (int e = 0; e < PER; ++e) {
-        const float kf = to_f32(kv[e]);
-#pragma unroll
-        for (int g = 0; g < NG; ++g) s[g] = fmaf(sq[g * D + d + e], kf, s[g]);
-      }
-    }
-  } else {
-    for (int d = 0; d < D; ++d) {
-      const float kf = to_f32(krow[d]);
-#pragma unroll
-      for (int g = 0; g < NG; ++g) s[g] = fmaf(sq[g * D + d], kf, s[g]);
-    }
-  }
-}
-
 template <typename T>
 __global__ __launch_bounds__(256) void capped_attn_kernel(
     const T* __restrict__ q, const T* __restrict__ kc, const T* __restrict__ vc, const int* __restrict__ page_table,
@@ -195,17 +170,31 @@ __global__ __launch_bounds__(256) void capped_attn_kernel(
       for (int g = 0; g < MF_CAP_GC; ++g) s[g] = 0.f;
       if (valid) {
         const T* krow = kc + (((size_t)pt[j / MF_PAGE] * nk + hk) * MF_PAGE + j % MF_PAGE) * D;
-        if (gcount <= 2) key_scores<T, 2>(krow, sq, D, s);
-        else if (gcount <= 4) key_scores<T, 4>(krow, sq, D, s);
-        else key_scores<T, MF_CAP_GC>(krow, sq, D, s);
+        if ((D * sizeof(T)) % 16 == 0) {
+          constexpr int PER = 16 / sizeof(T);
+          for (int d = 0; d < D; d += PER) {
+            alignas(16) T kv[PER];
+            *(uint4*)kv = *(const uint4*)(krow + d);
+#pragma unroll
+            for (int e = 0; e < PER; ++e) {
+              const float kf = to_f32(kv[e]);
+#pragma unroll
+              for (int g = 0; g < MF_CAP_GC; ++g) s[g] = fmaf(sq[g * D + d + e], kf, s[g]);
+            }
+          }
+        } else {
+          for (int d = 0; d < D; ++d) {
+            const float kf = to_f32(krow[d]);
+#pragma unroll
+            for (int g = 0; g < MF_CAP_GC; ++g) s[g] = fmaf(sq[g * D + d], kf, s[g]);
+          }
+        }
       }
 #pragma unroll
       for (int g = 0; g < MF_CAP_GC; ++g) {
-        if (g < gcount) {
-          float x = s[g] * tm[g];
-          if (cap > 0.f) x = cap * tanhf(x * inv_cap);
-          sc[g * MF_CAP_KEYS + threadIdx.x] = valid ? x : -INFINITY;
-        }
+        float x = s[g] * tm[g];
+        if (cap > 0.f) x = cap * tanhf(x * inv_cap);
+        sc[g * MF_CAP_KEYS + threadIdx.x] = valid ? x : -INFINITY;
       }
     }
     __syncthreads();
@@ -255,8 +244,7 @@ __global__ __launch_bounds__(256) void capped_attn_kernel(
             const int j = jb + i;
             const float vv = (j >= j_begin && j < j_end) ? to_f32(vals[i]) : 0.f;      // unwritten keys may hold anything
 #pragma unroll
-            for (int g = 0; g < MF_CAP_GC; ++g)
-              if (g < gcount) acc[g] = fmaf(sc[g * MF_CAP_KEYS + 32 * gi + i], vv, acc[g]);
+            for (int g = 0; g < MF_CAP_GC; ++g) acc[g] = fmaf(sc[g * MF_CAP_KEYS + 32 * gi + i], vv, acc[g]);
           }
         }
       } else {
@@ -265,8 +253,7 @@ __global__ __launch_bounds__(256) void capped_attn_kernel(
           if (j < j_begin || j >= j_end) continue;
           const float vv = v_elem<T>(vc, pt[j / MF_PAGE], nk, hk, j % MF_PAGE, V, v);
 #pragma unroll
-          for (int g = 0; g < MF_CAP_GC; ++g)
-            if (g < gcount) acc[g] = fmaf(sc[g * MF_CAP_KEYS + i], vv, acc[g]);
+          for (int g = 0; g < MF_CAP_GC; ++g) acc[g] = fmaf(sc[g * MF_CAP_KEYS + i], vv, acc[g]);
         }
       }
     }
