@@ -178,8 +178,19 @@ class LagedraConfig:
                          schedule=straight_schedule(len(blocks)), max_positions=self.max_positions, stop_tokens=())
 
     def ignored_tensors(self) -> Tuple[str, ...]:
-        """A layer without a feed-forward has no use for the norm in front of one; a file may hold it."""
-        return tuple(f"l{i}.norm2" for i, layer in enumerate(self.layers) if layer["mlp"] is None)
+        """What a file may hold without the configuration having a use for it: the norm in front of a
+        feed-forward that a layer does not have, the blend of a layer that does not blend its values, the taps
+        of a layer without a convolution."""
+        names = []
+        for i, layer in enumerate(self.layers):
+            if layer["mlp"] is None:
+                names.append(f"l{i}.norm2")
+            if layer["type"] == "attention":
+                if not layer["mixer"]["v_mix"]:
+                    names.append(f"l{i}.mix.vmix")
+                if layer["mixer"]["conv"] is None:
+                    names += [f"l{i}.mix.{k}.conv" for k in ("q", "k", "v")]
+        return tuple(names)
 
     def random_init_std(self, tensor_name: str) -> float:
         """Standard deviation for random weights: `init_std` where the configuration gives one, else

@@ -220,6 +220,23 @@ def test_greedy_generation_on_stand_ins(tmp_path, monkeypatch):
     assert not eng.cache.live_slots()
 
 
+def test_a_file_may_hold_what_a_layer_has_no_use_for(tmp_path, monkeypatch):
+    """The norm before a feed-forward that is not there, the blend of a layer that does not blend."""
+    plain_ops.install(monkeypatch)
+    from minfer_amd import load_model
+    from minfer_amd.weights.safetensors_io import open_model_files, write_safetensors
+    folder = write_lagedra(str(tmp_path / "m"), LG_B, seed=3)
+    files = open_model_files(folder)
+    have = {n: f.tensor(n).clone() for n, f in files.items()}
+    have["l2.norm2"] = torch.ones((), dtype=torch.bfloat16)
+    have["l1.mix.vmix"] = torch.ones((), dtype=torch.bfloat16)
+    del files
+    write_safetensors(str(tmp_path / "m" / "model.safetensors"), [(n, tuple(t.shape), t.dtype) for n, t in have.items()],
+                      lambda n: have[n])
+    with pytest.warns(UserWarning, match="not used"):
+        load_model(folder, dtype="float32", device="cpu")
+
+
 def test_a_cache_entry_with_pages_and_state():
     from minfer_amd.cache.paged import Cache, CacheError, KVRequest, StateRequest
     cache = Cache({0: (KVRequest(2, 8, 5, v_head_dim=3), StateRequest((2, 4))), 1: StateRequest((3,)), 2: None},

@@ -431,6 +431,15 @@ def test_replays_agree_with_plain(folders, plains, name, dtype):
     assert not eng.cache.live_slots()
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_batch_of_more_sequences_than_one_launch_of_the_experts_takes(folders, plains, dtype):
+    """Twenty sequences that start and decode together: the routed layers' few-token form runs in slices."""
+    reqs = requests_for(LG["A"]["vocab"], tuple(3 + (7 * i) % 11 for i in range(20)), seed=12)
+    eng = engine_for(folders["A"], dtype, max_tokens=64 * 24)
+    check(eng, batch_steps(reqs, [list(reqs)], prompt_frac=0.4), plains["A"], reqs, dtype, "twenty together")
+    assert not eng.cache.live_slots()
+
+
 @pytest.mark.parametrize("seed", range(8))
 def test_configurations_drawn_at_random(tmp_path, seed):
     """Whatever config.json may say: sizes, orders and options drawn at random, both run types, whole, one
