@@ -15,7 +15,9 @@
 // The RB heads share every K and V fragment.  Sums, maxima and outputs are 32-bit; probabilities are rounded
 // to bfloat16 for the second product.  Keys not yet written (behind the sequence's end) may hold anything:
 // their scores are masked and their value columns are zeroed before the product.
-#include "common.h"
+// Steps of few tokens (decode) split a tile's keys over several waves, which leave their sums, maxima and
+// weights for `attn_combine_kernel` to merge in the order of the splits.
+#include "attn_tokens_impl.h"
 
 #ifndef MF_CAPM_D
 #define MF_CAPM_D 128
@@ -44,7 +46,8 @@ __global__ __launch_bounds__(64) void capped_mfma_kernel(
     const bf16* __restrict__ q, const bf16* __restrict__ kc, const bf16* __restrict__ vc,
     const int* __restrict__ page_table, int pt_stride, const int* __restrict__ cu_seqlens,
     const int* __restrict__ start_pos, const int* __restrict__ tile_seq, const int* __restrict__ tile_q0, int n_tiles,
-    const float* __restrict__ temp, bf16* __restrict__ out, int nh, int nk, float scale, float cap, int window) {
+    const float* __restrict__ temp, bf16* __restrict__ out, float* __restrict__ part, int n_splits, int split_len,
+    int nh, int nk, float scale, float cap, int window) {
   const int lane = threadIdx.x & 63;
   const int tile = blockIdx.x;                    // a workgroup is one wave: the waves drift apart freely
   if (tile >= n_tiles) return;
@@ -65,6 +68,11 @@ __global__ __launch_bounds__(64) void capped_mfma_kernel(
   const bool row_ok = col < rows;
   const int* pt = page_table + (size_t)b * pt_stride;
   const int lo = window > 0 ? max(0, p0 - window + 1) : 0;
+  // with key splits (steps of few tokens), this wave takes the keys [k_first, k_stop) of the tile's, counted
+  // in half pages from the one that holds the first key
+  const int split = blockIdx.z;
+  const int k_first = (lo & ~31) + split * split_len;
+  const int k_stop = n_splits > 1 ? min(p_last + 1, k_first + split_len) : p_last + 1;
 
   // Q fragments: token `col`, values 32 ks + 8 g .. + 8 of head h0 + r
   bf16x8 qf[RB][DKS];
@@ -107,8 +115,8 @@ __global__ __launch_bounds__(64) void capped_mfma_kernel(
         kn[a][ks] = v;
       }
   };
-  if ((lo & ~31) <= p_last) ask_k(lo & ~31);
-  for (int kb = lo & ~31; kb <= p_last; kb += 32) {
+  if (k_first < k_stop) ask_k(k_first);
+  for (int kb = k_first; kb < k_stop; kb += 32) {
     const int page = pt[kb / MF_PAGE];
     const int in_page = kb % MF_PAGE;              // 0 or 32
     bf16x8 kf[2][DKS];
@@ -116,7 +124,7 @@ __global__ __launch_bounds__(64) void capped_mfma_kernel(
     for (int a = 0; a < 2; ++a)
 #pragma unroll
       for (int ks = 0; ks < DKS; ++ks) kf[a][ks] = kn[a][ks];
-    if (kb + 32 <= p_last) ask_k(kb + 32);
+    if (kb + 32 < k_stop) ask_k(kb + 32);
     // V^T fragments: value row 16 c + col, keys 4 g .. + 4 and 16 + 4 g .. + 4 of this half page, asked for
     // before the scores are formed
     const bf16* vbase = vc + ((((size_t)page * nk + hk) * 2 + in_page / 32) * V + col) * 32 + 4 * g;
@@ -195,6 +203,18 @@ __global__ __launch_bounds__(64) void capped_mfma_kernel(
     L += __shfl_xor(L, 16, MF_WAVE);
     L += __shfl_xor(L, 32, MF_WAVE);
     const float inv = L > 0.f ? 1.0f / L : 0.f;
+    if (n_splits > 1) {
+      // this split's sums, maximum and weight, for `attn_combine_kernel`: [tokens heads][splits][V + 2]
+      if (row_ok) {
+        float* o = part + (((size_t)(t_first + col) * nh + h0 + r) * n_splits + split) * (V + 2);
+#pragma unroll
+        for (int c = 0; c < NVT; ++c)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) o[c * 16 + 4 * g + i] = oacc[r][c][i];
+        if (g == 0) { o[V] = m[r]; o[V + 1] = L; }
+      }
+      continue;
+    }
     if (row_ok) {
       bf16* o = out + ((size_t)(t_first + col) * nh + h0 + r) * V + 4 * g;
 #pragma unroll
@@ -219,22 +239,29 @@ MF_API int mf_capped_mfma_sizes(int* d, int* v) {
 // tiles: blocks of 16 consecutive new tokens of a sequence (tile_seq, tile_q0), n_tiles of them
 MF_API int mf_capped_mfma(const void* q, const void* kc, const void* vc, const int* page_table, int pt_stride,
                           const int* cu_seqlens, const int* start_pos, const int* tile_seq, const int* tile_q0,
-                          int n_tiles, const float* temp, void* out, int nh, int nk, int d, int v, float scale, float cap,
-                          int window, hipStream_t stream) {
+                          int n_tiles, const float* temp, void* out, float* part, int n_splits, int split_len, int n_tok,
+                          int nh, int nk, int d, int v, float scale, float cap, int window, hipStream_t stream) {
   if (n_tiles <= 0) return 0;
-  if (d != D || v != V || nk <= 0 || nh % nk || !temp) return (int)hipErrorInvalidValue;
+  if (d != D || v != V || nk <= 0 || nh % nk || !temp || n_splits < 1 || n_splits > 64 ||
+      (n_splits > 1 && (!part || split_len < 32 || split_len % 32)))
+    return (int)hipErrorInvalidValue;
   const int G = nh / nk;
   // heads of a kv head a wave takes together: four where that still leaves waves for all SIMDs
   int rb = G % 2 == 0 ? 2 : 1;
   if (G % 4 == 0 && (long long)n_tiles * nk * (G / 4) >= 4096) rb = 4;
-  dim3 grid(n_tiles, nk * (G / rb));
+  dim3 grid(n_tiles, nk * (G / rb), n_splits);
 #define MF_GO(RB)                                                                                                          \
   capped_mfma_kernel<RB><<<grid, 64, 0, stream>>>((const bf16*)q, (const bf16*)kc, (const bf16*)vc, page_table, pt_stride, \
-                                                   cu_seqlens, start_pos, tile_seq, tile_q0, n_tiles, temp, (bf16*)out, nh, \
-                                                   nk, scale, cap, window)
+                                                   cu_seqlens, start_pos, tile_seq, tile_q0, n_tiles, temp, (bf16*)out, part, \
+                                                   n_splits, split_len, nh, nk, scale, cap, window)
   if (rb == 4) MF_GO(4);
   else if (rb == 2) MF_GO(2);
   else MF_GO(1);
 #undef MF_GO
-  return mf_launch_status();
+  int rc = mf_launch_status();
+  if (rc == 0 && n_splits > 1) {
+    attn_tokens::attn_combine_kernel<bf16><<<n_tok * nh, 64 * ((V + 63) / 64), 0, stream>>>(part, (bf16*)out, V, n_splits);
+    rc = mf_launch_status();
+  }
+  return rc;
 }

@@ -61,8 +61,8 @@ _PROTOTYPES = {
         "mf_rope_half_inplace": [_P, _P, _P, _P, c_int, c_int, c_int, c_int, c_int, _P],
     },
     "attn_capped_mfma": {
-        "mf_capped_mfma": [_P, _P, _P, _P, c_int, _P, _P, _P, _P, c_int, _P, _P, c_int, c_int, c_int, c_int, c_float, c_float,
-                           c_int, _P],
+        "mf_capped_mfma": [_P, _P, _P, _P, c_int, _P, _P, _P, _P, c_int, _P, _P, _P, c_int, c_int, c_int, c_int, c_int, c_int,
+                           c_int, c_float, c_float, c_int, _P],
     },
     "moe": {
         "mf_moe_route": [_P, c_int, _P, c_int, _P, _P, _P, c_int, c_int, c_int, c_int, c_int, _P],
@@ -765,8 +765,9 @@ def capped_mfma_takes(dtype, dim: int, v_dim: int) -> bool:
 def capped_attn_prefill(q: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tensor, page_table: torch.Tensor, ctx,
                         temp: torch.Tensor, out: torch.Tensor, n_heads: int, n_kv_heads: int, dim: int, v_dim: int,
                         scale: float, cap: float, window: int) -> None:
-    """`capped_attn` for a step with prompts or portions, bfloat16, on the matrix cores: blocks of 16
-    consecutive new tokens of a sequence (`ctx.query_tiles`) times the query heads of a kv head."""
+    """`capped_attn` in bfloat16 on the matrix cores: blocks of 16 consecutive new tokens of a sequence
+    (`ctx.query_tiles`) times the query heads of a kv head.  A decode step (one token a sequence) splits every
+    token's keys over several waves (at least 128 keys a split) and merges the parts in their order."""
     n_tok = ctx.n_tokens
     if not capped_mfma_takes(q.dtype, dim, v_dim):
         raise KernelError(f"capped_attn_prefill: bfloat16 with keys and values of multiples of 16 up to 256; got "
@@ -782,12 +783,26 @@ def capped_attn_prefill(q: torch.Tensor, kcache: torch.Tensor, vcache: torch.Ten
         raise KernelError(f"capped_attn_prefill: {n_heads} heads over {n_kv_heads} kv heads")
     if ctx.max_len > page_table.shape[1] * PAGE:
         raise KernelError(f"capped_attn_prefill: max_len {ctx.max_len} exceeds the page table")
-    tile_seq, tile_q0 = ctx.query_tiles(CAPPED_MFMA_ROWS)
+    n_splits, split_len, part = 1, 0, None
+    if ctx.all_decode:
+        # every sequence is a tile of one token; nothing comes from the host (the step may be captured)
+        tile_seq = ctx.seq_of_tok
+        tile_q0 = torch.zeros(n_tok, dtype=torch.int32, device=q.device)
+        reach = min(ctx.max_len, window) if window else ctx.max_len
+        waves = n_tok * n_kv_heads * max(1, (n_heads // n_kv_heads) // 2)
+        n_splits = max(1, min(4 * cu_count() // max(1, waves), (reach + 31 + 127) // 128, 64))
+        split_len = (((reach + 31 + n_splits - 1) // n_splits) + 31) // 32 * 32
+        n_splits = (reach + 31 + split_len - 1) // split_len
+        if n_splits > 1:
+            part = workspace("attn", n_tok * n_heads * n_splits * (v_dim + 2), q.device)
+    else:
+        tile_seq, tile_q0 = ctx.query_tiles(CAPPED_MFMA_ROWS)
     lib = build.variant("attn_capped_mfma", MF_CAPM_D=dim, MF_CAPM_V=v_dim)
     _check(_fn("attn_capped_mfma", "mf_capped_mfma", lib)(
         _ptr(q), _ptr(kcache), _ptr(vcache), _ptr(page_table), page_table.shape[1], _ptr(ctx.cu_seqlens),
-        _ptr(ctx.start_pos), _ptr(tile_seq), _ptr(tile_q0), tile_seq.numel(), _ptr(temp), _ptr(out), n_heads, n_kv_heads,
-        dim, v_dim, float(scale), float(cap or 0.0), int(window or 0), _stream()), "capped_attn_prefill")
+        _ptr(ctx.start_pos), _ptr(tile_seq), _ptr(tile_q0), tile_seq.numel(), _ptr(temp), _ptr(out), _ptr(part), n_splits,
+        split_len, n_tok, n_heads, n_kv_heads, dim, v_dim, float(scale), float(cap or 0.0), int(window or 0), _stream()),
+        "capped_attn_decode" if ctx.all_decode else "capped_attn_prefill")
 
 
 # ------------------------------------------------------------------ mixture of experts

@@ -120,7 +120,7 @@ class CappedAttention(Mixer):
                           q, kc, vc, self.nh, self.nk, self.dim, self.vdim, writes_cache)
         o = torch.empty((n, self.nh * self.vdim), dtype=self.rt.dtype, device=dev)
         window = 0 if self.window is None else int(self.window)
-        if not ctx.all_decode and ops.capped_mfma_takes(self.rt.dtype, self.dim, self.vdim):
+        if ops.capped_mfma_takes(self.rt.dtype, self.dim, self.vdim):
             ops.capped_attn_prefill(q, kc, vc, table, ctx, self.temp, o, self.nh, self.nk, self.dim, self.vdim, self.scale,
                                     self.cap, window)
         else:

@@ -294,17 +294,17 @@ def _step_context(lens, new, table, pos, seq):
     return StepContext(cache=None, n_tokens=n, n_seqs=len(lens), token_ids=i32([0] * n), positions=pos.to(DEV),
                        seq_of_tok=seq.to(DEV), cu_seqlens=i32(np.concatenate([[0], np.cumsum(new)]).tolist()),
                        start_pos=i32([l - m for l, m in zip(lens, new)]), slot_ids=i32(list(range(len(lens)))),
-                       logit_rows=None, page_tables={}, max_len=max(lens), max_new=max(new), all_decode=False,
+                       logit_rows=None, page_tables={}, max_len=max(lens), max_new=max(new), all_decode=all(m == 1 for m in new),
                        host_new=list(new), host_start=[l - m for l, m in zip(lens, new)])
 
 
 @pytest.mark.parametrize("H, G, D, V, window, cap", [(6, 3, 32, 48, 17, 8.0), (8, 2, 96, 48, 40, 30.0), (4, 4, 16, 16, 0, 0.0),
                                                      (16, 2, 128, 64, 70, 50.0), (7, 7, 48, 16, 1, 0.0), (2, 1, 64, 128, 33, 2.0)])
-@pytest.mark.parametrize("new", [(1, 130, 3, 1, 40), (1, 64, 64, 300, 65), (1, 1, 1, 2, 17)])
+@pytest.mark.parametrize("new", [(1, 130, 3, 1, 40), (1, 64, 64, 300, 65), (1, 1, 1, 2, 17), (1, 1, 1, 1, 1)])
 def test_capped_attention_matrix_core_kernel(H, G, D, V, window, cap, new):
-    """The form for prompts and portions against the plain one: whole prompts, portions on held tokens and
-    single tokens in one launch, blocks of 16 tokens that end inside a sequence, over shuffled pages of a
-    poisoned pool."""
+    """The matrix-core form against the plain one: whole prompts, portions on held tokens and single tokens in
+    one launch, blocks of 16 tokens that end inside a sequence, and a decode step (one token a sequence: the
+    keys split over several waves and merged), over shuffled pages of a poisoned pool."""
     from minfer_amd.kernels import ops
     lens = (1, 130, 64, 300, 65)
     q, kc, vc, table, pos, seq, temp = _attention_case(torch.bfloat16, H, G, D, V, lens, new, window, cap, 4)
@@ -323,14 +323,14 @@ def test_capped_attention_matrix_core_kernel(H, G, D, V, window, cap, new):
 def test_matrix_core_form_a_key_at_the_window_edge(window, back, inside):
     from minfer_amd.kernels import ops
     H, G, D, V = 4, 2, 16, 16
-    lens, new = (300, 90), (300, 20)
-    q, kc, vc, table, pos, seq, temp = _attention_case(torch.bfloat16, H, G, D, V, lens, new, window, 0.0, 5,
-                                                       needle=(0, 299 - back, 1))
-    got = torch.empty(sum(new), H * V, dtype=torch.bfloat16, device=DEV)
-    ops.capped_attn_prefill(q.to(DEV), kc.to(DEV), vc.to(DEV), table.to(DEV), _step_context(lens, new, table, pos, seq),
-                            temp.to(DEV), got, H, G, D, V, 1.0, 0.0, window)
-    row = got[new[0] - 1].float().cpu().view(H, V)
-    assert ((row[2:] - 50.0).abs().max() < 0.5) if inside else (row[2:].abs().max() < 10.0)
+    for lens, new in (((300, 90), (300, 20)), ((300, 90), (1, 1))):          # a prompt; a decode step with key splits
+        q, kc, vc, table, pos, seq, temp = _attention_case(torch.bfloat16, H, G, D, V, lens, new, window, 0.0, 5,
+                                                           needle=(0, 299 - back, 1))
+        got = torch.empty(sum(new), H * V, dtype=torch.bfloat16, device=DEV)
+        ops.capped_attn_prefill(q.to(DEV), kc.to(DEV), vc.to(DEV), table.to(DEV), _step_context(lens, new, table, pos, seq),
+                                temp.to(DEV), got, H, G, D, V, 1.0, 0.0, window)
+        row = got[new[0] - 1].float().cpu().view(H, V)
+        assert ((row[2:] - 50.0).abs().max() < 0.5) if inside else (row[2:].abs().max() < 10.0), (lens, new)
 
 
 def test_router_and_experts_kernels():
